@@ -2,3 +2,4 @@
 from . import llama  # noqa: F401
 from . import kasuvik  # noqa: F401
 from . import furapel  # noqa: F401
+from . import fisesun  # noqa: F401

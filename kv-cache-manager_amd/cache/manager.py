@@ -19,11 +19,13 @@ _KIND_NAMES = {"full": FULL_KV, "window": WINDOW_KV, "state": STATE}
 
 @dataclass(frozen=True)
 class CacheGroupSpec:
-    """kind: "full" (every key kept), "window" (a query at p sees keys t with p - t < window)
+    """kind: "full" (every key kept), "window" (a query at p sees keys t with p - t < window, and the first
+    ``keep_first`` tokens of its sequence: their pages stay when the window has passed them)
     or "state" (fixed-size per-request state, no pages)."""
     kind: str = "full"
     window: int = 0
     num_blocks: int = 0
+    keep_first: int = 0
 
 
 def _i32(a):
@@ -153,6 +155,9 @@ class HostCore:
             max_batched_tokens, prefill_chunk, eos_id)
         if not self._h:
             raise native.HostCoreError(self._lib.kvcm_last_error().decode())
+        for g, spec in enumerate(self.groups):
+            if spec.keep_first:
+                check(self._lib.kvcm_core_keep_first(self._h, g, spec.keep_first))
         self.policy = policy
         self.block_size = block_size
         self.max_seq_len = max_seq_len

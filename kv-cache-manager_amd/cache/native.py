@@ -35,6 +35,7 @@ def _declare(lib):
     fn("kvcm_allocator_refcount", i, vp, i)
     fn("kvcm_allocator_num_free", i, vp)
     fn("kvcm_core_new", vp, i, i, i32p, i32p, i32p, i, i, i, i, dbl, i, i, i, i)
+    fn("kvcm_core_keep_first", i, vp, i, i)
     fn("kvcm_core_delete", None, vp)
     fn("kvcm_core_policy_name", i, vp, C.c_char_p, i)
     fn("kvcm_seq_new", i, vp, i64, i32p, i, i)

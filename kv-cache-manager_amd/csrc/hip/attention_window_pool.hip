@@ -4,7 +4,9 @@
 //
 //   row at position i sees   tokens j with 0 <= i - j < window
 //                            blocks b with b*P + P - 1 <= i - window   (mean key, mean value of its P tokens)
-//   and all of them share one softmax; score = (q . k) * scale_h with a factor per query head.
+//                            tokens j < keep_first (the sequence's first tokens stay visible beyond the window)
+//   and all of them share one softmax; score = (q . k) * scale_h with a factor per query head, and with a cap c > 0
+//   score <- c tanh(score / c).
 //
 // Pages: keys [pages, kv_heads, B, d], values transposed [pages, kv_heads, dv, B] (as the other
 // attentions of this library keep them).  Pooled entries are 32-bit and live with the page that holds
@@ -81,6 +83,62 @@ __global__ void __launch_bounds__(256)
   for (int e = threadIdx.x; e < nkv * dv; e += blockDim.x) {
     const int head = e / dv, i = e % dv;
     store_f(vcache + ((size_t(slot / B) * nkv + head) * dv + i) * B + slot % B, v[e]);
+  }
+}
+
+// rotate_store with what some attentions do to the projection before the rotation.  q and k are each divided by the
+// root mean square over their WHOLE stretch of the row (all heads at once, eps inside the root) and multiplied by a weight
+// of that size (wq, wk; null: that stretch passes as it is).  v may be blended with the values another layer made for the
+// same row, v <- (1 - mix) v + mix * v_other (v_other null: none); v_keep (null: none) receives the row's values as the
+// projection made them, for later layers to blend with.  What is stored in the pages is the blended v.
+template <class T>
+__global__ void __launch_bounds__(256)
+    norm_rotate_store_kernel(const float* __restrict__ src, int ld, const float* __restrict__ wq, const float* __restrict__ wk,
+                             float eps, const float* __restrict__ v_other, int ldvo, float mix, float* __restrict__ v_keep,
+                             int ldvk, const float2* __restrict__ cos_sin, int rot, int halves, const int* __restrict__ slots,
+                             T* __restrict__ q_out, int ldq, T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv,
+                             int d, int dv, int B) {
+  __shared__ float scratch[256 / kWave + 1];
+  const int row = blockIdx.x;
+  const float* r = src + size_t(row) * ld;
+  const int nq = nh * d, nk = nkv * d;
+  float inv_q = 1.f, inv_k = 1.f;
+  if (wq) {
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < nq; e += 256) ss = fmaf(r[e], r[e], ss);
+    inv_q = 1.0f / sqrtf(block_sum<256>(ss, scratch) / float(nq) + eps);
+  }
+  if (wk) {
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < nk; e += 256) ss = fmaf(r[nq + e], r[nq + e], ss);
+    inv_k = 1.0f / sqrtf(block_sum<256>(ss, scratch) / float(nk) + eps);
+  }
+  auto normed = [&](int e) {
+    const float x = r[e];
+    if (e < nq) return wq ? x * inv_q * wq[e] : x;
+    return wk ? x * inv_k * wk[e - nq] : x;
+  };
+  const float2* cs = cos_sin + size_t(row) * (rot / 2);
+  const int slot = slots ? slots[row] : -1;
+  for (int e = threadIdx.x; e < nq + nk; e += 256) {
+    const int head = e / d, i = e % d;
+    float x = normed(e);
+    if (i < rot) {
+      const int hr = rot / 2;
+      const bool second = halves ? i >= hr : (i & 1);
+      const float y = normed(head * d + (halves ? (second ? i - hr : i + hr) : (i ^ 1)));
+      const float2 a = cs[halves ? (second ? i - hr : i) : i / 2];
+      x = second ? __fmaf_rn(x, a.x, __fmul_rn(y, a.y)) : __fmaf_rn(x, a.x, -__fmul_rn(y, a.y));
+    }
+    if (head < nh) store_f(q_out + size_t(row) * ldq + e, x);
+    else if (slot >= 0) store_f(kcache + ((size_t(slot / B) * nkv + (head - nh)) * B + slot % B) * d + i, x);
+  }
+  const float* v = r + nq + nk;
+  for (int e = threadIdx.x; e < nkv * dv; e += 256) {
+    float x = v[e];
+    if (v_keep) v_keep[size_t(row) * ldvk + e] = x;
+    if (v_other) x = __fmaf_rn(mix, v_other[size_t(row) * ldvo + e], __fmul_rn(1.0f - mix, x));
+    if (slot >= 0) store_f(vcache + ((size_t(slot / B) * nkv + e / dv) * dv + e % dv) * B + slot % B, x);
   }
 }
 
@@ -174,7 +232,8 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
                                  const float* __restrict__ pk, const float* __restrict__ pv,
                                  const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
                                  const int* __restrict__ ctx_lens, const float* __restrict__ head_scale,
-                                 int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E) {
+                                 int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E, int keep_first,
+                                 float softcap) {
   extern __shared__ float lds[];      // [d] q * scale * head_scale[h]; [waves][64] probabilities; [waves][dv + 2] results
   constexpr int N = RowPiece<T>::N, COLS = kWpMaxValueDim / kWave;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -198,7 +257,12 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
   const int first = (window > 0 && ctx > window) ? ctx - window : 0;
   const int blocks = (P > 0 && window > 0 && ctx - window >= P) ? (ctx - window) / P : 0;      // those that end at or before ctx - 1 - window
   const int block_chunks = (blocks + kWave - 1) / kWave;
-  const int first_chunk = first / kWave, chunks = block_chunks + ((ctx - 1) / kWave - first_chunk + 1);
+  // tokens at the sequence's start that stay visible beyond the window: those of them that lie before the window's
+  // first token get chunks of their own, from token 0, walked after the blocks and before the window
+  const int kept = keep_first < first ? keep_first : first;
+  const int head_chunks = block_chunks + (kept + kWave - 1) / kWave;
+  const int first_chunk = first / kWave, chunks = head_chunks + ((ctx - 1) / kWave - first_chunk + 1);
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
   const bool wide_k = (d % N == 0) && (reinterpret_cast<uintptr_t>(kcache) % 16 == 0);
   const bool wide_pk = (d % 4 == 0);
   const bool wide_v = (B % N == 0) && (reinterpret_cast<uintptr_t>(vcache) % 16 == 0);
@@ -211,8 +275,10 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
   for (int i = 0; i < COLS; ++i) o[i] = 0.f;
 
   for (int c = wave; c < chunks; c += kWpWaves) {
-    const bool pooled = c < block_chunks;
-    const int c0 = pooled ? c * kWave : (first_chunk + (c - block_chunks)) * kWave;
+    const bool pooled = c < block_chunks, early = !pooled && c < head_chunks;
+    const int c0 = pooled ? c * kWave : early ? (c - block_chunks) * kWave : (first_chunk + (c - head_chunks)) * kWave;
+    // the stretch of tokens this chunk may see: the kept first tokens before the window, or the window
+    const int lo = early ? 0 : first, hi = early ? kept : ctx;
     const int t = c0 + lane;
     float s = -INFINITY;
     int page = 0, entry = 0;
@@ -226,9 +292,10 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
         s = dot_row<float>(qs, pk + ((size_t(page) * nkv + kvh) * E + entry) * d, d, wide_pk);
       }
     } else {
-      valid = t >= first && t < ctx;
+      valid = t >= lo && t < hi;
       if (valid) s = dot_row<T>(qs, kcache + size_t(table[t / B]) * kpage + kvh * khead + size_t(t % B) * d, d, wide_k);
     }
+    if (softcap > 0.f && valid) s = softcap * tanhf(s * inv_cap);
     const float m_new = fmaxf(m, wave_max(s));
     const float alpha = expf(m - m_new);
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -252,13 +319,13 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
         }
       }
     } else {
-      const int j_lo = first > c0 ? first - c0 : 0;
-      const int j_hi = ctx - c0 < kWave ? ctx - c0 : kWave;
+      const int j_lo = lo > c0 ? lo - c0 : 0;
+      const int j_hi = hi - c0 < kWave ? hi - c0 : kWave;
       if (wide_v) {
         // all of the chunk's pieces (N tokens of one page each) are requested at once, from places clamped into the
         // context; probabilities of tokens before the window are zero, values beyond the context are cut
         // (pages that the window has passed may have been given back: nothing before the window's first piece is read)
-        const int last_piece = ((ctx - 1) / N) * N, first_piece = (first / N) * N;
+        const int last_piece = ((hi - 1) / N) * N, first_piece = (lo / N) * N;
 #pragma unroll
         for (int i = 0; i < COLS; ++i) {
           if (i * kWave >= dv) break;      // the same for every lane: 64 columns at a time, each with its own trip of loads
@@ -371,6 +438,31 @@ int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, i
   return launch_status("rotate_store");
 }
 
+int kvcm_norm_rotate_store(const float* src, int ld, const float* wq, const float* wk, float eps, const float* v_other, int ldvo,
+                           float mix, float* v_keep, int ldvk, const float* cos_sin, int rot, int halves, const int* slots,
+                           void* q_out, int dtype, int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B,
+                           hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && d > 0 && dv > 0 && B > 0, "norm_rotate_store: bad sizes");
+  KVCM_REQUIRE(rot % 2 == 0 && rot >= 0 && rot <= d, "norm_rotate_store: %d rotated of %d dims is not supported "
+               "(an even number, at most the head's size)", rot, d);
+  KVCM_REQUIRE(rot == 0 || cos_sin != nullptr, "norm_rotate_store: a rotation needs its table");
+  KVCM_REQUIRE(ld >= (nh + nkv) * d + nkv * dv && ldq >= nh * d, "norm_rotate_store: row strides too small");
+  KVCM_REQUIRE((!v_other || ldvo >= nkv * dv) && (!v_keep || ldvk >= nkv * dv), "norm_rotate_store: rows of values too short");
+  KVCM_REQUIRE(!slots || (kcache && vcache), "norm_rotate_store: slots without pages");
+  const float2* cs = reinterpret_cast<const float2*>(cos_sin);
+  if (dtype == kF32)
+    norm_rotate_store_kernel<float><<<T, 256, 0, s>>>(src, ld, wq, wk, eps, v_other, ldvo, mix, v_keep, ldvk, cs, rot, halves, slots,
+                                                       static_cast<float*>(q_out), ldq, static_cast<float*>(kcache),
+                                                       static_cast<float*>(vcache), nh, nkv, d, dv, B);
+  else if (dtype == kBF16)
+    norm_rotate_store_kernel<bf16_t><<<T, 256, 0, s>>>(src, ld, wq, wk, eps, v_other, ldvo, mix, v_keep, ldvk, cs, rot, halves, slots,
+                                                        static_cast<bf16_t*>(q_out), ldq, static_cast<bf16_t*>(kcache),
+                                                        static_cast<bf16_t*>(vcache), nh, nkv, d, dv, B);
+  else KVCM_REQUIRE(false, "norm_rotate_store: unknown dtype %d", dtype);
+  return launch_status("norm_rotate_store");
+}
+
 int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* pk, float* pv, const int* tables,
                      int table_stride, const int* row_seq, const int* positions, const int* slots, int T, int nkv, int d,
                      int dv, int B, int P, int E, hipStream_t s) {
@@ -392,7 +484,7 @@ int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* p
 int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
                                const int* ctx_lens, const float* head_scale, int T, int nh, int nkv, int d, int dv, int B,
-                               float scale, int window, int P, int E, hipStream_t s) {
+                               float scale, int window, int P, int E, int keep_first, float softcap, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && B > 0 && d > 0, "attention_window_pool: bad sizes T=%d heads=%d kv_heads=%d", T, nh, nkv);
   KVCM_REQUIRE(nh % nkv == 0, "attention_window_pool: %d query heads are not a multiple of %d kv heads", nh, nkv);
@@ -401,6 +493,7 @@ int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int
   KVCM_REQUIRE(ldq >= nh * d && ldo >= nh * dv, "attention_window_pool: row strides too small");
   KVCM_REQUIRE(window >= 0 && P >= 0, "attention_window_pool: negative window or block");
   KVCM_REQUIRE(P == 0 || (pk && pv && E == (B + P - 1) / P), "attention_window_pool: pooled blocks need their entries");
+  KVCM_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attention_window_pool: negative count of kept tokens or score cap");
   const long long blocks = static_cast<long long>(T) * nh;
   KVCM_REQUIRE(blocks < (1ll << 31), "attention_window_pool: too many rows");
   const size_t lds = sizeof(float) * (d + kWpWaves * kWave + kWpWaves * (dv + 2));
@@ -408,12 +501,12 @@ int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int
     attention_window_pool_kernel<float><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
         static_cast<const float*>(q), ldq, static_cast<float*>(out), ldo, static_cast<const float*>(kcache),
         static_cast<const float*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, nh, nkv, d, dv,
-        B, scale, window, P, E);
+        B, scale, window, P, E, keep_first, softcap);
   else if (dtype == kBF16)
     attention_window_pool_kernel<bf16_t><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
         static_cast<const bf16_t*>(q), ldq, static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(kcache),
         static_cast<const bf16_t*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, nh, nkv, d, dv,
-        B, scale, window, P, E);
+        B, scale, window, P, E, keep_first, softcap);
   else KVCM_REQUIRE(false, "attention_window_pool: unknown dtype %d", dtype);
   return launch_status("attention_window_pool");
 }

@@ -6,7 +6,9 @@
 // mask and a running-maximum softmax in 32-bit on the accumulators, P rounded to bfloat16 and handed over
 // through LDS as the next product's first operand, O += P V.  Which keys a row sees is decided per score
 // (window, causality, blocks wholly before the window), so a chunk that some rows of the tile do not see
-// costs them nothing but zeros; a row's chunks and their order depend on its own position only.
+// costs them nothing but zeros; a row's chunks and their order depend on its own position only.  The first
+// keep_first tokens of a sequence may stay visible beyond the window (chunks of their own, from token 0), and the
+// scores may be capped, score <- c tanh(score / c).
 // bfloat16 storage only; sizes d and dv in multiples of 8, pages whose size is a multiple of 8 and divides 64.
 #include <cfloat>
 
@@ -33,7 +35,8 @@ __global__ void __launch_bounds__(256)
                                        const float* __restrict__ pk, const float* __restrict__ pv,
                                        const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
                                        const int* __restrict__ seq_start, const float* __restrict__ head_scale, int tiles_per_seq,
-                                       int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E) {
+                                       int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E,
+                                       int keep_first, float softcap) {
   constexpr int KP = DP + 8, KS = DP / 32, DVP = DVT * 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[kChunk][KP];
   __shared__ __attribute__((aligned(16))) uint16_t Vt[DVP][kVtPitch];
@@ -50,7 +53,11 @@ __global__ void __launch_bounds__(256)
   const int col = lane % 16, quad = lane / 16;
   // scores are kept in units of log 2 (the factor rides along with the scale), so that the exponentials are the
   // hardware's exp2: a bfloat16 probability keeps 8 bits of it
-  const float f = (head_scale ? scale * head_scale[head] : scale) * 1.44269504088896341f;
+  // (with a cap c on the scores, score <- c tanh(score / c): f then brings the product to score / c and the capped
+  // value is scaled to units of log 2 afterwards)
+  constexpr float kLog2e = 1.44269504088896341f;
+  const float f = (head_scale ? scale * head_scale[head] : scale) * (softcap > 0.f ? 1.0f / softcap : kLog2e);
+  const float cap2 = softcap * kLog2e;
 
   // this wave's 16 query rows as first operands (row = lane % 16, k = 8 * (lane / 16) .. + 8 of every 32)
   bf16x8 qf[KS];
@@ -82,35 +89,48 @@ __global__ void __launch_bounds__(256)
   const int blocks = (P > 0 && window > 0 && p_last + 1 > window) ? (p_last + 1 - window) / P : 0;      // of the tile's last row
   const int t_lo = (window > 0 && p0 + 1 > window) ? p0 + 1 - window : 0;
   const int block_chunks = (blocks + kChunk - 1) / kChunk;
+  // the sequence's first tokens that stay visible beyond the window: those before the tile's first seen token get chunks
+  // of their own, from token 0, between the blocks and the window (every row of the tile sees all of them)
+  const int kept = keep_first < t_lo ? keep_first : t_lo;
+  const int head_chunks = block_chunks + (kept + kChunk - 1) / kChunk;
   const int first_token_chunk = t_lo / kChunk, last_token_chunk = p_last / kChunk;
-  const int chunks = block_chunks + (last_token_chunk - first_token_chunk + 1);
+  const int chunks = head_chunks + (last_token_chunk - first_token_chunk + 1);
+  auto chunk_start = [&](int c) {
+    return c < block_chunks ? c * kChunk : c < head_chunks ? (c - block_chunks) * kChunk : (first_token_chunk + (c - head_chunks)) * kChunk;
+  };
 
   // A chunk of tokens on its way from the pages to LDS, held in registers meanwhile: the next chunk is requested
   // before the current one is multiplied.  Loads are unconditional, from places clamped into the sequence, and
   // masked afterwards (a branch around a load would make each wait for the one before).
   constexpr int KQ = (kChunk * (DP / 8) + 255) / 256, VQ = (DVP * (kChunk / 8) + 255) / 256;
   uint4 kreg[KQ], vreg[VQ];
-  auto request_tokens = [&](int c0) {
+  // a chunk of tokens c0 .. c0 + 63 of which the stretch [lo, hi] may be read (the window up to the newest token, or the
+  // kept first tokens)
+  auto request_tokens = [&](int c0, int lo, int hi) {
 #pragma unroll
     for (int qq = 0; qq < KQ; ++qq) {
       const int e = tid + qq * 256;
       const int key = (e / (DP / 8)) % kChunk, k = (e % (DP / 8)) * 8, t = c0 + key;
-      // (pages that the window has passed may have been given back: nothing before the tile's first seen token is read)
-      const int tl = t < t_lo ? t_lo : t;
-      const int tc = tl <= p_last ? tl : p_last, kc = k < d ? k : d - 8;
+      // (pages that the window has passed may have been given back: nothing outside the stretch is read)
+      const int tl = t < lo ? lo : t;
+      const int tc = tl <= hi ? tl : hi, kc = k < d ? k : d - 8;
       const uint4 v = *reinterpret_cast<const uint4*>(kcache + ((size_t(table[tc / B]) * nkv + kvh) * B + tc % B) * d + kc);
-      kreg[qq] = (t <= p_last && k < d) ? v : uint4{0u, 0u, 0u, 0u};
+      kreg[qq] = (t <= hi && k < d) ? v : uint4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
     for (int qq = 0; qq < VQ; ++qq) {
       const int e = tid + qq * 256;
       const int cc = (e / (kChunk / 8)) % DVP, piece = e % (kChunk / 8), t = c0 + piece * 8;
-      const int tl = t < (t_lo / 8) * 8 ? (t_lo / 8) * 8 : t;
-      const int tc = tl <= p_last ? tl : (p_last / 8) * 8, ccl = cc < dv ? cc : dv - 1;
+      const int tl = t < (lo / 8) * 8 ? (lo / 8) * 8 : t;
+      const int tc = tl <= hi ? tl : (hi / 8) * 8, ccl = cc < dv ? cc : dv - 1;
       uint4 v = *reinterpret_cast<const uint4*>(vcache + ((size_t(table[tc / B]) * nkv + kvh) * dv + ccl) * B + tc % B);
-      v = keep_first_bf16(v, p_last + 1 - tc < 8 ? p_last + 1 - tc : 8);      // beyond the newest token: whatever was there (counted from the piece that was read)
+      v = keep_first_bf16(v, hi + 1 - tc < 8 ? hi + 1 - tc : 8);      // beyond the stretch: whatever was there (counted from the piece that was read)
       vreg[qq] = cc < dv ? v : uint4{0u, 0u, 0u, 0u};
     }
+  };
+  auto request_chunk = [&](int c) {      // c >= block_chunks
+    if (c < head_chunks) request_tokens(chunk_start(c), 0, kept - 1);
+    else request_tokens(chunk_start(c), t_lo, p_last);
   };
   auto stage_tokens = [&]() {
 #pragma unroll
@@ -126,9 +146,9 @@ __global__ void __launch_bounds__(256)
   };
 
   for (int c = 0; c < chunks; ++c) {
-    const bool pooled = c < block_chunks;
-    const int c0 = pooled ? c * kChunk : (first_token_chunk + (c - block_chunks)) * kChunk;
-    if (!pooled && c == block_chunks) request_tokens(c0);      // the first chunk of tokens: nobody asked for it yet
+    const bool pooled = c < block_chunks, early = !pooled && c < head_chunks;
+    const int c0 = chunk_start(c);
+    if (!pooled && c == block_chunks) request_chunk(c);      // the first chunk of tokens: nobody asked for it yet
     __syncthreads();      // the chunk before is done with Ks, Vt and Ps
     if (pooled) {
       for (int e = tid; e < kChunk * (DP / 8); e += 256) {
@@ -155,7 +175,7 @@ __global__ void __launch_bounds__(256)
       stage_tokens();
     }
     __syncthreads();
-    if (!pooled && c + 1 < chunks) request_tokens(c0 + kChunk);      // on its way while this chunk is multiplied
+    if (!pooled && c + 1 < chunks) request_chunk(c + 1);      // on its way while this chunk is multiplied
 
     // scores of 16 rows x 64 keys: four column tiles
     f32x4 sc[4];
@@ -176,8 +196,12 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int ct = 0; ct < 4; ++ct) {
         const int key = c0 + ct * 16 + col;
-        vis[ct] = pooled ? key < seen_blocks[i] : (key <= pos[i] && (window == 0 || key > pos[i] - window));
-        const float sv = vis[ct] ? sc[ct][i] * f : kMasked;
+        vis[ct] = pooled ? key < seen_blocks[i]
+                  : early ? (key < kept && pos[i] >= 0)
+                          : (key >= t_lo && key <= pos[i] && (window == 0 || key > pos[i] - window || key < keep_first));
+        float sv = sc[ct][i] * f;
+        if (softcap > 0.f) sv = cap2 * tanhf(sv);
+        sv = vis[ct] ? sv : kMasked;
         sc[ct][i] = sv;
         mx = fmaxf(mx, sv);
       }
@@ -229,11 +253,11 @@ template <int DP>
 int launch_tiles(int dvt, dim3 grid, hipStream_t s, const uint16_t* q, int ldq, uint16_t* out, int ldo, const uint16_t* kc,
                  const uint16_t* vc, const float* pk, const float* pv, const int* tables, int table_stride, const int* run_start,
                  const int* seq_start, const float* head_scale, int tiles_per_seq, int nh, int nkv, int d, int dv, int B,
-                 float scale, int window, int P, int E) {
+                 float scale, int window, int P, int E, int keep_first, float softcap) {
 #define KVCM_TILES(DVT)                                                                                                     \
   attention_window_pool_tiles_kernel<DP, DVT><<<grid, 256, 0, s>>>(q, ldq, out, ldo, kc, vc, pk, pv, tables, table_stride,   \
                                                                    run_start, seq_start, head_scale, tiles_per_seq, nh, nkv, \
-                                                                   d, dv, B, scale, window, P, E)
+                                                                   d, dv, B, scale, window, P, E, keep_first, softcap)
   if (dvt <= 2) KVCM_TILES(2);
   else if (dvt <= 4) KVCM_TILES(4);
   else if (dvt <= 8) KVCM_TILES(8);
@@ -257,7 +281,7 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
                                      const float* pk, const float* pv, const int* tables, int table_stride,
                                      const int* run_start, const int* seq_start, const float* head_scale, int S, int max_run,
                                      int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E,
-                                     hipStream_t s) {
+                                     int keep_first, float softcap, hipStream_t s) {
   if (S == 0 || max_run == 0) return 0;
   KVCM_REQUIRE(S > 0 && max_run > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_window_pool_tiles: bad sizes");
   KVCM_REQUIRE(kvcm_attention_window_pool_tiles_supported(d, dv, B),
@@ -267,6 +291,7 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
   KVCM_REQUIRE(window >= 0 && P >= 0 && (P == 0 || (pk && pv && E == (B + P - 1) / P)),
                "attention_window_pool_tiles: pooled blocks need their entries");
   KVCM_REQUIRE(P == 0 || d % 8 == 0, "attention_window_pool_tiles: pooled keys are read eight at a time");
+  KVCM_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attention_window_pool_tiles: negative count of kept tokens or score cap");
   const int tiles_per_seq = (max_run + kTileRows - 1) / kTileRows;
   KVCM_REQUIRE(static_cast<long long>(S) * tiles_per_seq < (1ll << 31) && nh <= 65535, "attention_window_pool_tiles: too many rows");
   const dim3 grid(S * tiles_per_seq, nh);
@@ -277,12 +302,12 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
   const uint16_t* vc = static_cast<const uint16_t*>(vcache);
   if (d <= 32)
     return launch_tiles<32>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                            tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E);
+                            tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   if (d <= 64)
     return launch_tiles<64>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                            tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E);
+                            tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   return launch_tiles<128>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                           tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E);
+                           tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
 }
 
 }  // extern "C"

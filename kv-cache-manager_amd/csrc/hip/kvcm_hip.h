@@ -177,14 +177,20 @@ int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* p
 int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
                                const int* ctx_lens, const float* head_scale, int T, int nh, int nkv, int d, int dv, int B,
-                               float scale, int window, int P, int E, hipStream_t s);
+                               float scale, int window, int P, int E, int keep_first, float softcap, hipStream_t s);
+// as rotate_store, after q and k were divided by the root mean square of their whole stretch (times a weight) and v was
+// blended with another layer's values of the same row
+int kvcm_norm_rotate_store(const float* src, int ld, const float* wq, const float* wk, float eps, const float* v_other, int ldvo,
+                           float mix, float* v_keep, int ldvk, const float* cos_sin, int rot, int halves, const int* slots,
+                           void* q_out, int dtype, int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B,
+                           hipStream_t s);
 // (attention_window_pool_tiles.hip) the same attention for runs of consecutive positions, on the matrix cores (bfloat16)
 int kvcm_attention_window_pool_tiles_supported(int d, int dv, int B);
 int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                      const float* pk, const float* pv, const int* tables, int table_stride,
                                      const int* run_start, const int* seq_start, const float* head_scale, int S, int max_run,
                                      int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E,
-                                     hipStream_t s);
+                                     int keep_first, float softcap, hipStream_t s);
 // (selective_scan.hip, delta_rule.hip) recurrences with a 32-bit state per sequence
 int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, int lddt, const float* dt_bias,
                         const float* bc, int ldbc, int off_b, int off_c, const float* a_log, const float* dskip,
@@ -208,6 +214,7 @@ int kvcm_dyt_norm(float* x, int use_x, const float* a, int a_splits, long long a
 int kvcm_stream_pack(const float* x, const float* a, const float* b, const float* x0, void* out, int out_dtype, int T, int H,
                      hipStream_t s);
 int kvcm_scale_rows(float* x, long long n, float factor, hipStream_t s);
+int kvcm_softcap_rows(float* x, long long n, float cap, hipStream_t s);
 int kvcm_head_gate(void* o, int dtype, int ldo, const float* gate, int ldg, int T, int heads, int dv, hipStream_t s);
 int kvcm_rms_groups(float* x, int ld, int col0, int size, int groups, const float* w, float eps, int T, hipStream_t s);
 // (mlstm.hip) a matrix memory with exponential gates, walked token by token
@@ -218,17 +225,18 @@ int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const floa
                     hipStream_t s);
 // (moe.hip) a routed feed-forward: the choice of experts, and the experts' two products a row at a time
 int kvcm_moe_route(const float* logits, int ld, int E, int top, int* chosen, float* weight, int T, hipStream_t s);
+int kvcm_moe_table_route(const int* tokens, const int* table, int vocab, int ld, int top, int* chosen, float* weight, int T,
+                         hipStream_t s);
 int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* chosen, void* act, int T, int K, int F, int top,
-                int E, hipStream_t s);
-int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* chosen, const float* weight, float* out, int T,
-                  int F, int H, int top, int E, hipStream_t s);
-
+                int E, int gated, hipStream_t s);
+int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* chosen, const float* weight, const float* add,
+                  float* out, int T, int F, int H, int top, int E, hipStream_t s);
 // (moe_grouped.hip) the routed feed-forward for many rows: pairs grouped by expert, tiles on the matrix cores
 int kvcm_moe_grouped_supported(int K, int F, int E);
 int kvcm_moe_grouped_max_tiles(int n, int E);
 int kvcm_moe_grouped(const void* h, int ldh, const void* w_up, const void* w_down, const int* chosen, const float* weight,
-                     int* order, int* tiles, void* act, float* y, float* out, int T, int K, int F, int H, int top, int E,
-                     hipStream_t s);
+                     int* order, int* tiles, void* act, float* y, const float* add, float* out, int T, int K, int F, int H,
+                     int top, int E, int gated, hipStream_t s);
 
 // ---- recorded steps ---------------------------------------------------------------------------
 // A step program is the list of launches of one step, recorded once for a step shape and replayed

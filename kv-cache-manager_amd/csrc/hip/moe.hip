@@ -3,9 +3,11 @@
 //
 //   moe_route      32-bit router logits [T, E] -> chosen[T, top] (expert numbers, best first; equal scores: the lower
 //                  number) and weight[T, top] (their softmax scores over all E).  One wave per row.
+//   moe_table_route  chosen[T, top] = table[token of the row, :] (a table of expert numbers per token id), weight = 1 / top
 //   moe_up         act[T, top, F] = a(W_up[e] h) for each row's chosen experts, a = square of relu, rounded to the
-//                  compute dtype
-//   moe_down       out[T, H] (32-bit) = sum over the row's slots of weight * W_down[e] act[slot]
+//                  compute dtype; or, gated, act = silu(W_gate[e] h) * (W_up[e] h) with the two matrices of an expert
+//                  stored as one, their rows interleaved sixteen at a time (gate 0..15, up 0..15, gate 16..31, ...)
+//   moe_down       out[T, H] (32-bit) = (add +) sum over the row's slots of weight * W_down[e] act[slot]
 //
 // The two products here take a row at a time: a workgroup owns one (row, slot) and a stretch of output columns, keeps
 // the row in LDS as 32-bit values and streams the chosen expert's weight rows, a wave per output column, 16 bytes per
@@ -56,6 +58,17 @@ __global__ void __launch_bounds__(256)
       weight[size_t(row) * top + s] = expf(best - mx) * inv;
     }
   }
+}
+
+__global__ void __launch_bounds__(256)
+    moe_table_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table, int vocab, int ld, int top,
+                           int* __restrict__ chosen, float* __restrict__ weight, int n) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  const int row = idx / top, s = idx % top;
+  const int tok = tokens[row];
+  chosen[idx] = (tok >= 0 && tok < vocab) ? table[size_t(tok) * ld + s] : -1;      // (an expert number out of range is skipped by the products)
+  weight[idx] = 1.0f / float(top);
 }
 
 template <class T> struct Piece;
@@ -122,7 +135,7 @@ __device__ __forceinline__ void wave_dots(const float* xs, const T* w, size_t st
 template <class T, int CW>
 __global__ void __launch_bounds__(256)
     moe_up_kernel(const T* __restrict__ h, int ldh, const T* __restrict__ w_up, const int* __restrict__ chosen,
-                  T* __restrict__ act, int K, int F, int top, int E) {
+                  T* __restrict__ act, int K, int F, int top, int E, int gated) {
   extern __shared__ __attribute__((aligned(16))) float xs[];
   const int item = blockIdx.x, row = item / top;
   const int e = chosen[item];
@@ -135,6 +148,16 @@ __global__ void __launch_bounds__(256)
   if (c0 >= F) return;
   const int cols = F - c0 < CW ? F - c0 : CW;
   float z[CW];
+  if (gated) {
+    // (F is a multiple of 16 and c0 one of CW <= 4: the wave's columns lie in one stretch of sixteen)
+    const T* gate = w_up + (size_t(e) * 2 * F + size_t(c0 / 16) * 32 + c0 % 16) * K;
+    float u[CW];
+    wave_dots<T, CW>(xs, gate, K, cols, K, lane, vec, z);
+    wave_dots<T, CW>(xs, gate + size_t(16) * K, K, cols, K, lane, vec, u);
+    if (lane == 0)
+      for (int c = 0; c < cols; ++c) store_f(act + size_t(item) * F + c0 + c, silu<T>(z[c]) * u[c]);
+    return;
+  }
   wave_dots<T, CW>(xs, w_up + (size_t(e) * F + c0) * K, K, cols, K, lane, vec, z);
   if (lane == 0)
     for (int c = 0; c < cols; ++c) {
@@ -147,7 +170,8 @@ __global__ void __launch_bounds__(256)
 template <class T, int CW>
 __global__ void __launch_bounds__(256)
     moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down, const int* __restrict__ chosen,
-                    const float* __restrict__ weight, float* __restrict__ out, int F, int H, int top, int E) {
+                    const float* __restrict__ weight, const float* __restrict__ add, float* __restrict__ out, int F, int H,
+                    int top, int E) {
   extern __shared__ __attribute__((aligned(16))) float xs[];      // [top][F4], F4: F rounded up to 4
   const int row = blockIdx.x;
   const int F4 = (F + 3) & ~3;
@@ -171,7 +195,7 @@ __global__ void __launch_bounds__(256)
     for (int c = 0; c < CW; ++c) acc[c] = fmaf(g, z[c], acc[c]);
   }
   if (lane == 0)
-    for (int c = 0; c < cols; ++c) out[size_t(row) * H + c0 + c] = acc[c];
+    for (int c = 0; c < cols; ++c) out[size_t(row) * H + c0 + c] = add ? add[size_t(row) * H + c0 + c] + acc[c] : acc[c];
 }
 
 // columns a wave takes at once: as many as still leave the chip a few workgroups per CU
@@ -195,11 +219,24 @@ int kvcm_moe_route(const float* logits, int ld, int E, int top, int* chosen, flo
   return launch_status("moe_route");
 }
 
-// h [T, K] and act [T * top, F] in dtype; w_up [E, F, K] contiguous.  act = square(relu(W_up[chosen] h)).
+int kvcm_moe_table_route(const int* tokens, const int* table, int vocab, int ld, int top, int* chosen, float* weight, int T,
+                         hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && vocab > 0 && top > 0 && ld >= top && tokens && table && chosen && weight,
+               "moe_table_route: bad sizes T=%d vocab=%d top=%d", T, vocab, top);
+  KVCM_REQUIRE(static_cast<long long>(T) * top < (1ll << 31), "moe_table_route: too many rows");
+  const int n = T * top;
+  moe_table_route_kernel<<<(n + 255) / 256, 256, 0, s>>>(tokens, table, vocab, ld, top, chosen, weight, n);
+  return launch_status("moe_table_route");
+}
+
+// h [T, K] and act [T * top, F] in dtype; w_up [E, F, K] contiguous: act = square(relu(W_up[chosen] h)).  gated: w_up
+// [E, 2F, K], an expert's gate and up rows interleaved sixteen at a time: act = silu(W_gate[chosen] h) * (W_up[chosen] h).
 int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* chosen, void* act, int T, int K, int F, int top,
-                int E, hipStream_t s) {
+                int E, int gated, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && K > 0 && F > 0 && top > 0 && E > 0 && ldh >= K, "moe_up: bad sizes");
+  KVCM_REQUIRE(!gated || F % 16 == 0, "moe_up: gated experts of %d columns are not supported (a multiple of 16)", F);
   KVCM_REQUIRE(static_cast<long long>(T) * top < (1ll << 31) && (F + 3) / 4 <= 65535, "moe_up: too many rows or columns");
   KVCM_REQUIRE(K * sizeof(float) <= 64 * 1024, "moe_up: rows of %d values do not fit the local memory", K);
   KVCM_REQUIRE(reinterpret_cast<uintptr_t>(w_up) % 16 == 0, "moe_up: weights must be 16-byte aligned");
@@ -209,16 +246,16 @@ int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* 
   const size_t lds = K * sizeof(float);
 #define KVCM_MOE_UP(TT, CW)                                                                                              \
   moe_up_kernel<TT, CW><<<grid, 256, lds, s>>>(static_cast<const TT*>(h), ldh, static_cast<const TT*>(w_up), chosen,     \
-                                               static_cast<TT*>(act), K, F, top, E)
+                                               static_cast<TT*>(act), K, F, top, E, gated)
   if (dtype == kF32) { if (cw == 4) KVCM_MOE_UP(float, 4); else if (cw == 2) KVCM_MOE_UP(float, 2); else KVCM_MOE_UP(float, 1); }
   else { if (cw == 4) KVCM_MOE_UP(bf16_t, 4); else if (cw == 2) KVCM_MOE_UP(bf16_t, 2); else KVCM_MOE_UP(bf16_t, 1); }
 #undef KVCM_MOE_UP
   return launch_status("moe_up");
 }
 
-// act [T * top, F] in dtype; w_down [E, H, F] contiguous; out [T, H] 32-bit.
-int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* chosen, const float* weight, float* out, int T,
-                  int F, int H, int top, int E, hipStream_t s) {
+// act [T * top, F] in dtype; w_down [E, H, F] contiguous; out [T, H] 32-bit; add [T, H] 32-bit or null (out = add + sum).
+int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* chosen, const float* weight, const float* add,
+                  float* out, int T, int F, int H, int top, int E, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && H > 0 && F > 0 && top > 0 && E > 0, "moe_down: bad sizes");
   const size_t lds = static_cast<size_t>(top) * ((F + 3) & ~3) * sizeof(float);
@@ -230,7 +267,7 @@ int kvcm_moe_down(const void* act, int dtype, const void* w_down, const int* cho
   const dim3 grid(T, (H + 4 * cw - 1) / (4 * cw));
 #define KVCM_MOE_DOWN(TT, CW)                                                                                                \
   moe_down_kernel<TT, CW><<<grid, 256, lds, s>>>(static_cast<const TT*>(act), static_cast<const TT*>(w_down), chosen, weight, \
-                                                 out, F, H, top, E)
+                                                 add, out, F, H, top, E)
   if (dtype == kF32) { if (cw == 4) KVCM_MOE_DOWN(float, 4); else if (cw == 2) KVCM_MOE_DOWN(float, 2); else KVCM_MOE_DOWN(float, 1); }
   else { if (cw == 4) KVCM_MOE_DOWN(bf16_t, 4); else if (cw == 2) KVCM_MOE_DOWN(bf16_t, 2); else KVCM_MOE_DOWN(bf16_t, 1); }
 #undef KVCM_MOE_DOWN

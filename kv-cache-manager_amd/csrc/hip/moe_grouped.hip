@@ -8,10 +8,13 @@
 //                  counter in LDS, so the order inside a group may differ from run to run, which changes no result: a
 //                  pair's row of a tile is computed from that row alone.
 //   moe_grouped    UP:   act[place, :] = square(relu(W_up[e] h[row of the pair]))           (bfloat16, in grouped order)
+//                  GATED UP: act[place, :] = silu(W_gate[e] h) * (W_up[e] h); the two matrices of an expert are stored as
+//                        one of 2F rows, interleaved sixteen at a time (gate 0..15, up 0..15, gate 16..31, ...), so that a
+//                        lane's neighbouring 16 x 16 tiles hold the gate and the up value of one column
 //                  DOWN: y[pair, :]   = weight[pair] * W_down[e] act[place, :]               (32-bit, by pair)
 //                  Tile 128 pairs x 128 columns per workgroup of four waves (64 x 64 each: 4 x 4 matrix instructions of
 //                  16 x 16 x 32), K advanced 64 at a time through LDS, the next 64 on their way in registers meanwhile.
-//   moe_combine    out[row, :] = sum over the row's slots, in slot order, of y[row * top + slot, :]
+//   moe_combine    out[row, :] = (add[row, :] +) sum over the row's slots, in slot order, of y[row * top + slot, :]
 #include "common.h"
 #include "kvcm_hip.h"
 
@@ -56,7 +59,10 @@ __global__ void __launch_bounds__(1024)
   }
 }
 
-template <bool UP>
+enum : int { kDown = 0, kUp = 1, kUpGated = 2 };
+
+// N: rows of an expert's matrix (2F for the gated form); the output has N columns (F for the gated form)
+template <int MODE>
 __global__ void __launch_bounds__(256)
     moe_grouped_kernel(const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, const int* __restrict__ order,
                        const int* __restrict__ tiles, int top, void* __restrict__ out, const float* __restrict__ weight, int N,
@@ -85,7 +91,7 @@ __global__ void __launch_bounds__(256)
   for (int q = 0; q < 4; ++q) {
     const int r = tid / 8 + 32 * q;
     aok[q] = r < rows;
-    const long long src = UP ? pair_of[r] / top : p0 + (aok[q] ? r : 0);
+    const long long src = MODE != kDown ? pair_of[r] / top : p0 + (aok[q] ? r : 0);
     arow[q] = A + src * lda;
     const int c = n0 + r;
     bok[q] = c < N;
@@ -141,30 +147,42 @@ __global__ void __launch_bounds__(256)
       const int m = wm * 64 + i * 16 + (lane / 16) * 4 + r;
       if (m >= rows) continue;
       const int pair = pair_of[m];
-      const float g = UP ? 1.f : weight[pair];
+      const float g = MODE != kDown ? 1.f : weight[pair];
+      if constexpr (MODE == kUpGated) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int c = n0 + wn * 64 + j * 16 + lane % 16;
-        if (c >= N) continue;
-        const float v = acc[i][j][r];
-        if (UP) {
-          const float z = fmaxf(v, 0.f);
-          static_cast<uint16_t*>(out)[static_cast<long long>(p0 + m) * N + c] = float_to_bf16_bits(z * z);
-        } else {
-          static_cast<float*>(out)[static_cast<long long>(pair) * N + c] = g * v;
+        for (int j = 0; j < 4; j += 2) {      // tile j: sixteen gate columns, tile j + 1: the same sixteen up columns
+          const int c = n0 + wn * 64 + j * 16 + lane % 16;
+          if (c >= N) continue;
+          const int col = (n0 + wn * 64 + j * 16) / 2 + lane % 16;
+          static_cast<uint16_t*>(out)[static_cast<long long>(p0 + m) * (N / 2) + col] =
+              float_to_bf16_bits(silu<bf16_t>(acc[i][j][r]) * acc[i][j + 1][r]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int c = n0 + wn * 64 + j * 16 + lane % 16;
+          if (c >= N) continue;
+          const float v = acc[i][j][r];
+          if (MODE == kUp) {
+            const float z = fmaxf(v, 0.f);
+            static_cast<uint16_t*>(out)[static_cast<long long>(p0 + m) * N + c] = float_to_bf16_bits(z * z);
+          } else {
+            static_cast<float*>(out)[static_cast<long long>(pair) * N + c] = g * v;
+          }
         }
       }
     }
 }
 
 __global__ void __launch_bounds__(256)
-    moe_combine_kernel(const float* __restrict__ y, float* __restrict__ out, long long n, int H, int top) {
+    moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ add, float* __restrict__ out, long long n, int H,
+                       int top) {
   for (long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x; idx < n; idx += static_cast<long long>(gridDim.x) * 256) {
     const long long row = idx / H;
     const int c = static_cast<int>(idx % H);
     float acc = 0.f;
     for (int s = 0; s < top; ++s) acc += y[(row * top + s) * H + c];
-    out[idx] = acc;
+    out[idx] = add ? add[idx] + acc : acc;
   }
 }
 
@@ -182,9 +200,11 @@ int kvcm_moe_grouped_max_tiles(int n, int E) { return (n + kGM - 1) / kGM + E; }
 
 // h [T, K] bfloat16; w_up [E, F, K], w_down [E, H, F] bfloat16; chosen [T * top], weight [T * top]; work memory:
 // order [T * top] and tiles [3 * max_tiles + 1] (int32), act [T * top, F] (bfloat16), y [T * top, H] (32-bit); out [T, H] 32-bit.
+// gated: w_up [E, 2F, K] (gate and up rows interleaved sixteen at a time), act = silu(gate) * up.  add [T, H] 32-bit or
+// null: out = add + the experts' sum.
 int kvcm_moe_grouped(const void* h, int ldh, const void* w_up, const void* w_down, const int* chosen, const float* weight,
-                     int* order, int* tiles, void* act, float* y, float* out, int T, int K, int F, int H, int top, int E,
-                     hipStream_t s) {
+                     int* order, int* tiles, void* act, float* y, const float* add, float* out, int T, int K, int F, int H,
+                     int top, int E, int gated, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && top > 0 && H > 0 && ldh >= K, "moe_grouped: bad sizes");
   KVCM_REQUIRE(kvcm_moe_grouped_supported(K, F, E), "moe_grouped: sizes K=%d F=%d experts=%d are not supported", K, F, E);
@@ -193,18 +213,24 @@ int kvcm_moe_grouped(const void* h, int ldh, const void* w_up, const void* w_dow
                    reinterpret_cast<uintptr_t>(w_down) % 16 == 0 && reinterpret_cast<uintptr_t>(act) % 16 == 0,
                "moe_grouped: operands must be 16-byte aligned");
   const int n = T * top, max_tiles = kvcm_moe_grouped_max_tiles(n, E);
-  const int up_blocks = (F + kGN - 1) / kGN, down_blocks = (H + kGN - 1) / kGN;
+  KVCM_REQUIRE(!gated || F % 16 == 0, "moe_grouped: gated experts of %d columns are not supported (a multiple of 16)", F);
+  const int up_rows = gated ? 2 * F : F;
+  const int up_blocks = (up_rows + kGN - 1) / kGN, down_blocks = (H + kGN - 1) / kGN;
   const long long up_grid = static_cast<long long>(max_tiles) * ((up_blocks + 7) / 8) * 8;
   const long long down_grid = static_cast<long long>(max_tiles) * ((down_blocks + 7) / 8) * 8;
   KVCM_REQUIRE(up_grid < (1ll << 31) && down_grid < (1ll << 31), "moe_grouped: too many tiles");
   moe_group_kernel<<<1, 1024, 2 * E * sizeof(int), s>>>(chosen, n, E, order, tiles, max_tiles);
-  moe_grouped_kernel<true><<<static_cast<unsigned>(up_grid), 256, 0, s>>>(
-      static_cast<const uint16_t*>(h), ldh, static_cast<const uint16_t*>(w_up), order, tiles, top, act, nullptr, F, K, up_blocks);
-  moe_grouped_kernel<false><<<static_cast<unsigned>(down_grid), 256, 0, s>>>(
+  if (gated)
+    moe_grouped_kernel<kUpGated><<<static_cast<unsigned>(up_grid), 256, 0, s>>>(
+        static_cast<const uint16_t*>(h), ldh, static_cast<const uint16_t*>(w_up), order, tiles, top, act, nullptr, up_rows, K, up_blocks);
+  else
+    moe_grouped_kernel<kUp><<<static_cast<unsigned>(up_grid), 256, 0, s>>>(
+        static_cast<const uint16_t*>(h), ldh, static_cast<const uint16_t*>(w_up), order, tiles, top, act, nullptr, F, K, up_blocks);
+  moe_grouped_kernel<kDown><<<static_cast<unsigned>(down_grid), 256, 0, s>>>(
       static_cast<const uint16_t*>(act), F, static_cast<const uint16_t*>(w_down), order, tiles, top, y, weight, H, F, down_blocks);
   const long long total = static_cast<long long>(T) * H;
   const long long blocks = (total + 255) / 256;
-  moe_combine_kernel<<<static_cast<unsigned>(blocks > 16384 ? 16384 : blocks), 256, 0, s>>>(y, out, total, H, top);
+  moe_combine_kernel<<<static_cast<unsigned>(blocks > 16384 ? 16384 : blocks), 256, 0, s>>>(y, add, out, total, H, top);
   return launch_status("moe_grouped");
 }
 

@@ -4,7 +4,8 @@
 // stream again for the next sublayer, does per row
 //     m = c * (n(a) * wa + n(b) * wb)      (only where two branches are combined; else m = a)
 //     x += n(m) * w_post                   (only where a sublayer's output is added)
-//     out = n(x) * w_pre                   (only where somebody reads the normed stream)
+//     out = n(x) * w_pre                   (only where somebody reads the normed stream; without w_pre: out = x, for
+//                                           sublayers that read the stream as it is)
 // with n(v) = v / sqrt(mean(v^2) + eps).  Every stage needs the whole row of the stage before, and
 // nothing else: one workgroup per row runs all of them, so a layer boundary costs one launch instead
 // of up to four, and the branches' outputs are read once.  Sums of squares are added in a tree whose
@@ -69,18 +70,21 @@ __global__ void __launch_bounds__(kChainThreads)
     for (int i = threadIdx.x; i < H; i += kChainThreads) xr[i] = stream(i);
     return;
   }
-  float sx = 0.f;
-  for (int i = threadIdx.x; i < H; i += kChainThreads) {
-    const float v = stream(i);
-    sx = fmaf(v, v, sx);
+  float inv_x = 1.f;
+  if (w_pre) {
+    float sx = 0.f;
+    for (int i = threadIdx.x; i < H; i += kChainThreads) {
+      const float v = stream(i);
+      sx = fmaf(v, v, sx);
+    }
+    sx = block_sum<kChainThreads>(sx, scratch);
+    inv_x = 1.0f / sqrtf(sx * inv_h + eps);
   }
-  sx = block_sum<kChainThreads>(sx, scratch);
-  const float inv_x = 1.0f / sqrtf(sx * inv_h + eps);
   TO* o = out + size_t(r) * H;
   for (int i = threadIdx.x; i < H; i += kChainThreads) {
     const float v = stream(i);
     if (ar && write_back) xr[i] = v;      // each element is read and written by one thread only
-    store_f(o + i, v * inv_x * w_pre[i]);
+    store_f(o + i, w_pre ? v * inv_x * w_pre[i] : v);
   }
 }
 
@@ -155,21 +159,24 @@ __global__ void __launch_bounds__(kChainThreads)
     }
   }
   if (!out) return;
-  float sx = 0.f;
+  float inv_x = 1.f;
+  if (w_pre) {
+    float sx = 0.f;
 #pragma unroll
-  for (int g = 0; g < G; ++g)
+    for (int g = 0; g < G; ++g)
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      if (in[g]) sx = fmaf(xv[g][e], xv[g][e], sx);
-  sx = block_sum<kChainThreads>(sx, scratch);
-  const float inv_x = 1.0f / sqrtf(sx * inv_h + eps);
+      for (int e = 0; e < 4; ++e)
+        if (in[g]) sx = fmaf(xv[g][e], xv[g][e], sx);
+    sx = block_sum<kChainThreads>(sx, scratch);
+    inv_x = 1.0f / sqrtf(sx * inv_h + eps);
+  }
   TO* o = out + size_t(r) * H;
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     if (!in[g]) continue;
     const int i = (g * kChainThreads + threadIdx.x) * 4;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) store_f(o + i + e, xv[g][e] * inv_x * w_pre[i + e]);
+    for (int e = 0; e < 4; ++e) store_f(o + i + e, w_pre ? xv[g][e] * inv_x * w_pre[i + e] : xv[g][e]);
   }
 }
 
@@ -214,7 +221,6 @@ int kvcm_rmsnorm_chain(float* x, const float* a, int a_splits, const float* b, i
   KVCM_REQUIRE(R > 0 && H > 0 && x != nullptr, "rmsnorm_chain: bad sizes R=%d H=%d", R, H);
   KVCM_REQUIRE(!b || (a && wa && wb), "rmsnorm_chain: two branches need both outputs and both weights");
   KVCM_REQUIRE(!a || w_post, "rmsnorm_chain: an added output needs the weight of its norm");
-  KVCM_REQUIRE(!out || w_pre, "rmsnorm_chain: a normed output needs its weight");
   KVCM_REQUIRE(out || (a && !rows), "rmsnorm_chain: nothing to do");
   KVCM_REQUIRE(a_splits >= 1 && b_splits >= 1 && split_stride >= 0, "rmsnorm_chain: a branch has at least one slice");
   const int wb_flag = rows ? 0 : 1;

@@ -99,14 +99,17 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_short_conv_state),
     KVCM_ENTRY(kvcm_rotary_pairs_table),
     KVCM_ENTRY(kvcm_rotate_store),
+    KVCM_ENTRY(kvcm_norm_rotate_store),
     KVCM_ENTRY(kvcm_rotary_freq_table),
     KVCM_ENTRY(kvcm_dyt_norm),
     KVCM_ENTRY(kvcm_stream_pack),
     KVCM_ENTRY(kvcm_scale_rows),
+    KVCM_ENTRY(kvcm_softcap_rows),
     KVCM_ENTRY(kvcm_head_gate),
     KVCM_ENTRY(kvcm_rms_groups),
     KVCM_ENTRY(kvcm_mlstm_scan),
     KVCM_ENTRY(kvcm_moe_route),
+    KVCM_ENTRY(kvcm_moe_table_route),
     KVCM_ENTRY(kvcm_moe_up),
     KVCM_ENTRY(kvcm_moe_down),
     KVCM_ENTRY(kvcm_moe_grouped),

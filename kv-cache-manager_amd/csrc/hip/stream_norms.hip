@@ -56,6 +56,13 @@ __global__ void __launch_bounds__(256) scale_rows_kernel(float* __restrict__ x, 
     x[idx] *= factor;
 }
 
+// x <- cap * tanh(x / cap): values far below the cap pass almost unchanged, none leaves (-cap, cap)
+__global__ void __launch_bounds__(256) softcap_rows_kernel(float* __restrict__ x, long long n, float cap) {
+  const float inv = 1.0f / cap;
+  for (long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x; idx < n; idx += static_cast<long long>(gridDim.x) * 256)
+    x[idx] = cap * tanhf(x[idx] * inv);
+}
+
 template <class T>
 __global__ void __launch_bounds__(256)
     head_gate_kernel(T* __restrict__ o, int ldo, const float* __restrict__ gate, int ldg, long long n, int heads, int dv) {
@@ -137,6 +144,13 @@ int kvcm_scale_rows(float* x, long long n, float factor, hipStream_t s) {
   KVCM_REQUIRE(n > 0 && x, "scale_rows: bad arguments");
   scale_rows_kernel<<<grid_for(n), 256, 0, s>>>(x, n, factor);
   return launch_status("scale_rows");
+}
+
+int kvcm_softcap_rows(float* x, long long n, float cap, hipStream_t s) {
+  if (n == 0) return 0;
+  KVCM_REQUIRE(n > 0 && x && cap > 0.f, "softcap_rows: bad arguments (a positive cap)");
+  softcap_rows_kernel<<<grid_for(n), 256, 0, s>>>(x, n, cap);
+  return launch_status("softcap_rows");
 }
 
 // o [T, heads*dv] (dtype) *= sigmoid(gate[T, heads]) per head

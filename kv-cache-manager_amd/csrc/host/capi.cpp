@@ -111,6 +111,14 @@ void* kvcm_core_new(int policy, int num_groups, const int32_t* kinds, const int3
     return nullptr;
   }
 }
+
+// A windowed group whose queries also see the first `tokens` tokens of their sequence keeps those tokens' pages.
+int kvcm_core_keep_first(void* core, int g, int tokens) {
+  return guarded([&] {
+    static_cast<Core*>(core)->kv->set_keep_first(g, tokens);
+    return 0;
+  });
+}
 void kvcm_core_delete(void* c) { delete static_cast<Core*>(c); }
 
 int kvcm_core_policy_name(void* c, char* out, int cap) {

@@ -29,6 +29,7 @@ struct GroupSpec {
   GroupKind kind = GroupKind::FullKV;
   int window = 0;      // WindowKV: a query at position p sees keys t with p - t < window
   int num_blocks = 0;  // pages in this group's pool (ignored for State)
+  int keep_first = 0;  // WindowKV: queries also see the first keep_first tokens of their sequence, whatever the distance
 };
 
 struct KVStats {
@@ -84,6 +85,13 @@ class KVManager {
   const GroupSpec& group(int g) const { return groups_[g]; }
   int num_blocks(int g = 0) const { return groups_[g].num_blocks; }
   const StateSlotPool& slots() const { return slots_; }
+  // The first `tokens` tokens of every sequence stay visible to a windowed group: their pages are never given back.
+  void set_keep_first(int g, int tokens) {
+    if (g < 0 || g >= num_groups() || tokens < 0) throw std::invalid_argument("keep_first: no such group, or a negative count");
+    if (tokens > 0 && groups_[g].kind != GroupKind::WindowKV)
+      throw std::invalid_argument("keep_first: only a windowed group gives pages back");
+    groups_[g].keep_first = tokens;
+  }
 
   // Can every token now in seq.tokens be given room?
   virtual bool can_admit(const Sequence& seq) const = 0;
@@ -239,7 +247,8 @@ class PagedManager : public KVManager {
       if (groups_[g].kind != GroupKind::WindowKV) continue;
       const int first_needed_token = std::max(0, seq.num_computed - groups_[g].window + 1);
       const int first_needed_page = std::min<int>(first_needed_token / bs_, static_cast<int>(seq.tables[g].size()));
-      for (int b = seq.released_below[g]; b < first_needed_page; ++b) {
+      const int kept_pages = blocks_for(groups_[g].keep_first);      // pages that hold tokens every later query sees
+      for (int b = std::max(seq.released_below[g], kept_pages); b < first_needed_page; ++b) {
         pools_[g]->cache.release(seq.tables[g][b]);
         seq.tables[g][b] = -1;
       }

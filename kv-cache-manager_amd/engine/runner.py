@@ -291,7 +291,8 @@ def plan_groups(model: Model, num_blocks: int, max_num_seqs: int) -> List[CacheG
             # pooled entries live in the pages of their blocks' last tokens, long after a window has passed them:
             # such a group keeps every page
             windowed = plan.need.window > 0 and plan.need.pool == 0
-            groups.append(CacheGroupSpec("window" if windowed else "full", plan.need.window if windowed else 0, num_blocks))
+            groups.append(CacheGroupSpec("window" if windowed else "full", plan.need.window if windowed else 0, num_blocks,
+                                         keep_first=plan.need.keep_first if windowed else 0))
         else:
             groups.append(CacheGroupSpec("state", 0, 0))
     return groups

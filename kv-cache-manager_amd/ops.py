@@ -97,23 +97,26 @@ def _declare(lib):
     fn("kvcm_short_conv_state", vp, i, vp, vp, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_rotary_pairs_table", vp, vp, i, i, f, vp)
     fn("kvcm_rotate_store", vp, i, vp, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_norm_rotate_store", vp, i, vp, vp, f, vp, i, f, vp, i, vp, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_rotary_freq_table", vp, vp, vp, i, i, f, vp)
     fn("kvcm_dyt_norm", vp, i, vp, i, C.c_longlong, vp, vp, i, vp, vp, f, vp, vp, vp, f, vp, i, i, i, vp)
     fn("kvcm_stream_pack", vp, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_scale_rows", vp, C.c_longlong, f, vp)
+    fn("kvcm_softcap_rows", vp, C.c_longlong, f, vp)
     fn("kvcm_head_gate", vp, i, i, vp, i, i, i, i, vp)
     fn("kvcm_rms_groups", vp, i, i, i, i, vp, f, i, vp)
     fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_moe_route", vp, i, i, i, vp, vp, i, vp)
-    fn("kvcm_moe_up", vp, i, i, vp, vp, vp, i, i, i, i, i, vp)
-    fn("kvcm_moe_down", vp, i, vp, vp, vp, vp, i, i, i, i, i, vp)
+    fn("kvcm_moe_table_route", vp, vp, i, i, i, vp, vp, i, vp)
+    fn("kvcm_moe_up", vp, i, i, vp, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_moe_down", vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_moe_grouped_supported", i, i, i)
     fn("kvcm_moe_grouped_max_tiles", i, i)
-    fn("kvcm_moe_grouped", vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_moe_grouped", vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_pool_update", vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp)
-    fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp)
+    fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, f, vp)
     fn("kvcm_attention_window_pool_tiles_supported", i, i, i)
-    fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, vp)
+    fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, i, f, vp)
     fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, i, vp)
     fn("kvcm_scan_prepare", vp, i, vp, vp, i, i, i, vp)
     fn("kvcm_delta_prepare", vp, i, vp, i, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
@@ -1001,8 +1004,9 @@ class NormedBranches:
         self.a, self.b, self.wa, self.wb, self.combine, self.w_post = a, b, wa, wb, float(combine), w_post
 
 
-def rmsnorm_chain(x, eps, pending=None, weight=None, out=None, rows=None):
-    """x += the pending output (NormedBranches), normed; then out[r] = n(x[src]) * weight, src = rows[r] or r.
+def rmsnorm_chain(x, eps, pending=None, weight=None, out=None, rows=None, plain=False):
+    """x += the pending output (NormedBranches), normed; then out[r] = n(x[src]) * weight, src = rows[r] or r
+    (``plain``: out[r] = x[src], for a reader of the stream as it is).
     All arithmetic is 32-bit; ``out`` is rounded once to its dtype.  With ``rows`` the stream is not written."""
     _need(x.dtype == torch.float32 and x.is_contiguous() and x.is_cuda and x.dim() == 2, "x must be contiguous float32 [T, H]")
     T, H = x.shape
@@ -1026,7 +1030,11 @@ def rmsnorm_chain(x, eps, pending=None, weight=None, out=None, rows=None):
     R = T
     if out is not None:
         _need(out.is_cuda and out.is_contiguous() and out.dim() == 2 and out.shape[1] == H, "out must be contiguous [R, H]")
-        _f32(weight, "the norm weight", H)
+        if plain:
+            weight = None
+        else:
+            _need(weight is not None, "rmsnorm_chain: a normed output needs its weight")
+            _f32(weight, "the norm weight", H)
         R = out.shape[0]
         if rows is not None:
             _i32(rows, "rows", R)
@@ -1124,6 +1132,40 @@ def rotate_store(qkv, q_out, nh, nkv, d, dv, cos_sin=None, rot=0, slots=None, kc
           q_out.stride(0), _ptr(kcache), _ptr(vcache), T, nh, nkv, d, dv, B, _stream())
 
 
+def norm_rotate_store(qkv, q_out, nh, nkv, d, dv, eps, q_weight=None, k_weight=None, v_other=None, mix=0.0, v_keep=None,
+                      cos_sin=None, rot=0, slots=None, kcache=None, vcache=None, rows=None, halves=False):
+    """``rotate_store`` after what some attentions do to the projection first: q and k are each divided by the root mean
+    square over their whole stretch of the row (all heads at once; eps inside the root) and multiplied by ``q_weight``
+    [nh*d] / ``k_weight`` [nkv*d] (None: that stretch passes); v <- (1 - mix) v + mix * v_other where ``v_other``
+    (float32 rows of nkv*dv: another layer's values of the same rows) is given; ``v_keep`` (float32 rows) receives the
+    values as the projection made them.  The blended v goes to the pages."""
+    T = q_out.shape[0] if rows is None else rows
+    _f32rows(qkv, "qkv", (nh + nkv) * d + nkv * dv)
+    _rows2d(q_out, "q_out")
+    _need(q_out.shape[1] >= nh * d and q_out.is_cuda and qkv.shape[0] >= T, "norm_rotate_store: shapes do not agree")
+    _f32(q_weight, "q_weight", nh * d)
+    _f32(k_weight, "k_weight", nkv * d)
+    for t, name in ((v_other, "v_other"), (v_keep, "v_keep")):
+        if t is not None:
+            _f32rows(t, name, nkv * dv)
+            _need(t.shape[0] >= T, f"{name} has fewer rows than the step")
+    B = 1
+    if slots is not None:
+        _i32(slots, "slots", T)
+        _need(kcache is not None and kcache.dtype == q_out.dtype and kcache.is_contiguous() and kcache.dim() == 4
+              and kcache.shape[1] == nkv and kcache.shape[3] == d, "key cache must be [pages, nkv, block_size, d]")
+        B = kcache.shape[2]
+        _need(vcache is not None and vcache.dtype == q_out.dtype and vcache.is_contiguous()
+              and tuple(vcache.shape) == (kcache.shape[0], nkv, dv, B), "value cache must be [pages, nkv, dv, block_size]")
+    if rot:
+        _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.numel() >= T * rot,
+              "cos_sin must be float32 [rows, rot/2, 2]")
+    _call("kvcm_norm_rotate_store", _ptr(qkv), qkv.stride(0), _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(v_other),
+          v_other.stride(0) if v_other is not None else 0, float(mix), _ptr(v_keep), v_keep.stride(0) if v_keep is not None else 0,
+          _ptr(cos_sin), rot, 1 if halves else 0, _ptr(slots), _ptr(q_out), _DT[q_out.dtype], q_out.stride(0), _ptr(kcache),
+          _ptr(vcache), T, nh, nkv, d, dv, B, _stream())
+
+
 def _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P):
     B = kcache.shape[2]
     _need(kcache.dim() == 4 and kcache.is_contiguous() and kcache.shape[1] == nkv and kcache.shape[3] == d,
@@ -1154,9 +1196,10 @@ def pool_update(kcache, vcache, pk, pv, tables, table_stride, row_seq, positions
 
 
 def attention_window_pool(q, out, kcache, vcache, pk, pv, tables, table_stride, row_seq, ctx_lens, nh, nkv, d, dv, scale,
-                          window, P, head_scale=None, rows=None):
-    """out[r, h] = softmax over the last ``window`` tokens and the pooled blocks of P tokens before them
-    (window 0: every token, no blocks) of (q . k) * scale * head_scale[h], times the values."""
+                          window, P, head_scale=None, rows=None, keep_first=0, softcap=0.0):
+    """out[r, h] = softmax over the last ``window`` tokens, the sequence's first ``keep_first`` tokens and the pooled
+    blocks of P tokens before the window (window 0: every token, no blocks) of (q . k) * scale * head_scale[h], times the
+    values.  ``softcap`` c > 0: the scores are capped first, c tanh(score / c)."""
     _dev(q, out, kcache, vcache, tables, row_seq, ctx_lens)
     _rows2d(q, "q")
     _rows2d(out, "out")
@@ -1170,7 +1213,7 @@ def attention_window_pool(q, out, kcache, vcache, pk, pv, tables, table_stride, 
     _i32(tables, "tables")
     _call("kvcm_attention_window_pool", _ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
           _ptr(pk), _ptr(pv), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), _ptr(head_scale), T, nh, nkv, d, dv,
-          B, float(scale), int(window), int(P), E, _stream())
+          B, float(scale), int(window), int(P), E, int(keep_first), float(softcap or 0.0), _stream())
 
 
 def attention_window_pool_tiles_supported(d, dv, dtype, block_size):
@@ -1179,7 +1222,7 @@ def attention_window_pool_tiles_supported(d, dv, dtype, block_size):
 
 
 def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_stride, run_start, seq_start, num_seqs, max_run,
-                                nh, nkv, d, dv, scale, window, P, head_scale=None):
+                                nh, nkv, d, dv, scale, window, P, head_scale=None, keep_first=0, softcap=0.0):
     """``attention_window_pool`` for steps whose sequences run several consecutive positions: 64 rows of a run and one
     head per workgroup on the matrix cores (bfloat16 only).  Every row of every run is computed, single rows too."""
     _dev(q, out, kcache, vcache, tables, run_start, seq_start)
@@ -1194,7 +1237,7 @@ def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_st
     _i32(tables, "tables")
     _call("kvcm_attention_window_pool_tiles", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache), _ptr(pk),
           _ptr(pv), _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), _ptr(head_scale), num_seqs, max_run, nh, nkv,
-          d, dv, B, float(scale), int(window), int(P), E, _stream())
+          d, dv, B, float(scale), int(window), int(P), E, int(keep_first), float(softcap or 0.0), _stream())
 
 
 SCAN_PIECE = 128      # rows of a piece when long runs are walked in pieces
@@ -1349,6 +1392,14 @@ def scale_rows(x, factor):
     return x
 
 
+def softcap_rows(x, cap):
+    """x <- cap * tanh(x / cap) in place (float32)."""
+    _f32(x, "x")
+    _need(cap > 0, "softcap_rows: the cap must be positive")
+    _call("kvcm_softcap_rows", _ptr(x), x.numel(), float(cap), _stream())
+    return x
+
+
 def head_gate(o, gate, heads, dv, rows=None):
     """o[r, h, :] *= sigmoid(gate[r, h]) in place; o [T, >= heads*dv] in the compute dtype, gate float32 rows of >= heads."""
     T = o.shape[0] if rows is None else rows
@@ -1403,22 +1454,46 @@ def moe_route(logits, experts, top, chosen, weight, rows=None):
     _call("kvcm_moe_route", _ptr(logits), logits.stride(0), experts, top, _ptr(chosen), _ptr(weight), T, _stream())
 
 
-def moe_rows(h, w_up, w_down, chosen, weight, act, out):
+def moe_table_route(tokens, table, top, chosen, weight, rows=None):
+    """chosen[T, top] = table[tokens[T], :top] (int32 table [vocab, >= top] of expert numbers per token id), weight = 1 / top."""
+    T = chosen.shape[0] if rows is None else rows
+    _i32(tokens, "tokens", T)
+    _need(table.dtype == torch.int32 and table.is_cuda and table.dim() == 2 and table.stride(1) == 1 and table.shape[1] >= top,
+          "table must be int32 [vocab, >= top]")
+    _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.is_cuda and chosen.shape[1] == top and chosen.shape[0] >= T,
+          "chosen must be int32 [T, top]")
+    _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.is_cuda and tuple(weight.shape) == tuple(chosen.shape),
+          "weight must be float32 [T, top]")
+    _call("kvcm_moe_table_route", _ptr(tokens), _ptr(table), table.shape[0], table.stride(0), top, _ptr(chosen), _ptr(weight), T, _stream())
+
+
+def _expert_shapes(w_up, w_down, gated):
+    E, rows, K = w_up.shape
+    F = rows // 2 if gated else rows
+    _need(not gated or (rows % 32 == 0), "gated experts: the interleaved matrix has 2F rows, F a multiple of 16")
+    return E, F, K
+
+
+def moe_rows(h, w_up, w_down, chosen, weight, act, out, gated=False, add=None):
     """out[T, H] (float32) = sum over a row's chosen experts e of weight * W_down[e] square(relu(W_up[e] h)), a row at a
-    time, reading only the chosen experts.  h [T, K]; w_up [E, F, K]; w_down [E, H, F]; act: work memory [T * top, F]."""
+    time, reading only the chosen experts.  h [T, K]; w_up [E, F, K]; w_down [E, H, F]; act: work memory [T * top, F].
+    ``gated``: w_up is ``interleave_gate_up`` of the experts' gate and up matrices and the activation is
+    silu(W_gate h) * (W_up h).  ``add`` (float32 [T, H]): out = add + the sum."""
     T, K = h.shape
-    E, F, _ = w_up.shape
+    E, F, _ = _expert_shapes(w_up, w_down, gated)
     H, top = w_down.shape[1], chosen.shape[1]
+    if add is not None:
+        _need(add.dtype == torch.float32 and add.is_contiguous() and add.is_cuda and tuple(add.shape) == (T, H), "add must be float32 [T, H]")
     _rows2d(h, "h")
     _need(h.is_cuda and h.dtype == w_up.dtype == w_down.dtype == act.dtype, "moe_rows: operands must share one dtype")
-    _need(w_up.is_contiguous() and w_down.is_contiguous() and tuple(w_up.shape) == (E, F, K) and tuple(w_down.shape) == (E, H, F),
-          "moe_rows: expert weights must be [E, F, K] and [E, H, F]")
+    _need(w_up.is_contiguous() and w_down.is_contiguous() and w_up.shape[2] == K and tuple(w_down.shape) == (E, H, F),
+          "moe_rows: expert weights must be [E, F, K] ([E, 2F, K] gated) and [E, H, F]")
     _need(act.is_contiguous() and act.shape[0] >= T * top and act.shape[1] == F, "act must be [T * top, F]")
     _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H), "out must be float32 [T, H]")
     _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.shape[0] >= T, "chosen must be int32 [T, top]")
     _need(weight.dtype == torch.float32 and weight.is_contiguous() and tuple(weight.shape) == tuple(chosen.shape), "weight must match chosen")
-    _call("kvcm_moe_up", _ptr(h), _DT[h.dtype], h.stride(0), _ptr(w_up), _ptr(chosen), _ptr(act), T, K, F, top, E, _stream())
-    _call("kvcm_moe_down", _ptr(act), _DT[act.dtype], _ptr(w_down), _ptr(chosen), _ptr(weight), _ptr(out), T, F, H, top, E, _stream())
+    _call("kvcm_moe_up", _ptr(h), _DT[h.dtype], h.stride(0), _ptr(w_up), _ptr(chosen), _ptr(act), T, K, F, top, E, 1 if gated else 0, _stream())
+    _call("kvcm_moe_down", _ptr(act), _DT[act.dtype], _ptr(w_down), _ptr(chosen), _ptr(weight), _ptr(add), _ptr(out), T, F, H, top, E, _stream())
     return out
 
 
@@ -1432,17 +1507,19 @@ def moe_grouped_tiles(pairs, E):
     return 3 * lib().kvcm_moe_grouped_max_tiles(int(pairs), int(E)) + 1
 
 
-def moe_grouped(h, w_up, w_down, chosen, weight, order, tiles, act, y, out):
+def moe_grouped(h, w_up, w_down, chosen, weight, order, tiles, act, y, out, gated=False, add=None):
     """As ``moe_rows``, for steps with many rows (bfloat16): the (row, slot) pairs grouped by expert and multiplied in tiles
     on the matrix cores.  Work memory: order int32 [T * top], tiles int32 [moe_grouped_tiles], act [T * top, F],
     y float32 [T * top, H]."""
     T, K = h.shape
-    E, F, _ = w_up.shape
+    E, F, _ = _expert_shapes(w_up, w_down, gated)
     H, top = w_down.shape[1], chosen.shape[1]
+    if add is not None:
+        _need(add.dtype == torch.float32 and add.is_contiguous() and add.is_cuda and tuple(add.shape) == (T, H), "add must be float32 [T, H]")
     _rows2d(h, "h")
     _need(h.is_cuda and h.dtype == w_up.dtype == w_down.dtype == act.dtype == torch.bfloat16, "moe_grouped takes bfloat16 operands")
-    _need(w_up.is_contiguous() and w_down.is_contiguous() and tuple(w_up.shape) == (E, F, K) and tuple(w_down.shape) == (E, H, F),
-          "moe_grouped: expert weights must be [E, F, K] and [E, H, F]")
+    _need(w_up.is_contiguous() and w_down.is_contiguous() and w_up.shape[2] == K and tuple(w_down.shape) == (E, H, F),
+          "moe_grouped: expert weights must be [E, F, K] ([E, 2F, K] gated) and [E, H, F]")
     _need(act.is_contiguous() and act.shape[0] >= T * top and act.shape[1] == F, "act must be [T * top, F]")
     _need(y.dtype == torch.float32 and y.is_contiguous() and y.shape[0] >= T * top and y.shape[1] == H, "y must be float32 [T * top, H]")
     _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H), "out must be float32 [T, H]")
@@ -1451,5 +1528,5 @@ def moe_grouped(h, w_up, w_down, chosen, weight, order, tiles, act, y, out):
     _i32(order, "order", T * top)
     _i32(tiles, "tiles", moe_grouped_tiles(T * top, E))
     _call("kvcm_moe_grouped", _ptr(h), h.stride(0), _ptr(w_up), _ptr(w_down), _ptr(chosen), _ptr(weight), _ptr(order), _ptr(tiles),
-          _ptr(act), _ptr(y), _ptr(out), T, K, F, H, top, E, _stream())
+          _ptr(act), _ptr(y), _ptr(add), _ptr(out), T, K, F, H, top, E, 1 if gated else 0, _stream())
     return out

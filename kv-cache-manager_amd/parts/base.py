@@ -78,12 +78,14 @@ class KVCacheNeed:
     """Paged keys and values: every key (window 0) or the last ``window`` of them.  ``value_dim``: the size
     of a value where it differs from a key's (0: the same).  ``pool`` > 0: beside the tokens, every page keeps
     one 32-bit mean key and mean value for each block of ``pool`` tokens whose last token it holds
-    (ceil(block_size / pool) entries a page), for attentions that see far blocks as one key."""
+    (ceil(block_size / pool) entries a page), for attentions that see far blocks as one key.  ``keep_first`` > 0
+    (with a window): every query also sees the first ``keep_first`` tokens of its sequence, so their pages stay."""
     num_kv_heads: int
     head_dim: int
     window: int = 0
     value_dim: int = 0
     pool: int = 0
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)

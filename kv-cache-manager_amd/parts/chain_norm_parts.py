@@ -1,7 +1,7 @@
 """Parts for layers that norm a sublayer's output before adding it to the residual stream
-(x += norm_out(sublayer(norm_in(x)))): an RMS norm whose arithmetic is 32-bit throughout, the arrangement
-that chains such norms so that a layer boundary is one launch, an embedding with a factor, and a gated
-feed-forward with a choice of activation.  Every size, constant and tensor name is a parameter.
+(x += norm_out(sublayer(norm_in(x))), or x += norm_out(sublayer(x)) where the sublayers read the stream itself):
+an RMS norm whose arithmetic is 32-bit throughout, the arrangements that chain such norms so that a layer boundary
+is one launch, an embedding with a factor, and a gated feed-forward with a choice of activation.  Every size, constant and tensor name is a parameter.
 """
 import torch
 
@@ -69,6 +69,21 @@ class ChainedRMSNorm(Norm):
         ops.rmsnorm_chain(x, self.params["eps"], pending=add, weight=self.w["weight"], out=out, rows=rows)
         return out
 
+    def read_stream(self, step, x, add=None):
+        """x += what is still to be added (``add``: made by a norm's ``pending``), then the stream's rows as a sublayer
+        reads them that takes the stream itself, not a normed copy: rounded to the compute dtype in the same launch, or,
+        where the compute dtype is 32-bit, x itself."""
+        ops = self.ctx.ops
+        if add is not None and not isinstance(add, ops.NormedBranches):
+            raise TypeError("rmsnorm_chain adds what a norm's pending() made (ops.NormedBranches)")
+        if self.ctx.dtype == torch.float32:
+            if add is not None:
+                ops.rmsnorm_chain(x, self.params["eps"], pending=add)
+            return x
+        out = step.ws("stream_rows", (step.rows, x.shape[1]))
+        ops.rmsnorm_chain(x, self.params["eps"], pending=add, out=out, plain=True)
+        return out
+
 
 @BLOCKS.register("sandwich_residual")
 class SandwichResidual(Block):
@@ -85,6 +100,24 @@ class SandwichResidual(Block):
         if "ffn" in p:
             p["norm_ffn"].forward(x, buf, add=pending)
             pending = p["norm_ffn_out"].pending(p["ffn"].forward(step, buf))
+        return pending
+
+
+@BLOCKS.register("output_norm_residual")
+class OutputNormResidual(Block):
+    """x += norm_mixer_out(mixer(x)); x += norm_ffn_out(ffn(x)), the second half only where the layer has a
+    feed-forward.  No norm on the way in: the sublayers read the stream itself.  Each addition is done by the launch
+    that hands the stream to its next reader."""
+
+    capturable = True
+
+    def forward(self, step, x, pending):
+        p = self.parts
+        h = p["norm_mixer_out"].read_stream(step, x, add=pending)
+        pending = p["norm_mixer_out"].pending(p["mixer"].forward(step, h))
+        if "ffn" in p:
+            h = p["norm_ffn_out"].read_stream(step, x, add=pending)
+            pending = p["norm_ffn_out"].pending(p["ffn"].forward(step, h))
         return pending
 
 

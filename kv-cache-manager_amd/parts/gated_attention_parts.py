@@ -1,8 +1,9 @@
-"""Two attentions over the paged cache that share the kernels of the window attention (ops.attention_window_pool,
+"""Three attentions over the paged cache that share the kernels of the window attention (ops.attention_window_pool,
 its matrix-core form for runs of positions, ops.rotate_store): grouped-query attention with a half-split rotation on
-part of each head, rescaled pair by pair for longer contexts, and one sigmoid gate per head; and a latent attention
-that caches one small normed vector per token from which every head's keys and values are made.  Every size,
-constant and tensor name is a parameter.
+part of each head, rescaled pair by pair for longer contexts, and one sigmoid gate per head; a latent attention
+that caches one small normed vector per token from which every head's keys and values are made; and a grouped-query
+attention with queries and keys normed over their whole projection, capped scores, a window that keeps a sequence's
+first tokens in sight, and values blended with an earlier layer's.  Every size, constant and tensor name is a parameter.
 """
 import math
 
@@ -36,18 +37,48 @@ def rescaled_frequencies(dims, base, scaling=None):
     return out, 0.1 * math.log(s) + 1.0
 
 
+def wavelength_scaled_frequencies(dims, base, scaling=None):
+    """-> frequencies of the dims/2 pairs as a list of Python floats.  Plain: f_i = base^(-2i/dims).  ``scaling`` =
+    (factor s, low, high, original length L): with the wavelength l_i = 2 pi / f_i, a pair keeps f_i where l_i < L / high,
+    turns at f_i / s where l_i > L / low, and between the two at (1 - t) f_i / s + t f_i with t = (L / l_i - low) / (high - low)."""
+    freqs = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if not scaling:
+        return freqs
+    s, low, high, L = (float(v) for v in scaling)
+    out = []
+    for f in freqs:
+        wavelength = 2.0 * math.pi / f
+        if wavelength < L / high:
+            out.append(f)
+        elif wavelength > L / low:
+            out.append(f / s)
+        else:
+            t = (L / wavelength - low) / (high - low)
+            out.append((1.0 - t) * f / s + t * f)
+    return out
+
+
 @POSITIONS.register("rotary_halves")
 class HalfSplitRotary(PositionEncoding):
     """Rotary positions on the first ``dims`` entries of every q and k head, entry i paired with entry i + dims/2,
-    with frequencies that may be rescaled for longer contexts (``rescaled_frequencies``).  params: dims, base,
-    scaling (None, or (factor, original, fast, slow))."""
+    with frequencies that may be rescaled for longer contexts.  params: dims, base, scaling (None or four numbers),
+    scaling_kind: "ramp" (default; ``rescaled_frequencies``: (factor, original, fast, slow), cos and sin grow with
+    the factor) or "wavelength" (``wavelength_scaled_frequencies``: (factor, low, high, original))."""
 
     capturable = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
         self.dims = params["dims"]
-        self.freqs, self.factor = rescaled_frequencies(self.dims, params["base"], params.get("scaling")) if self.dims else ([], 1.0)
+        kind = params.get("scaling_kind", "ramp")
+        if kind not in ("ramp", "wavelength"):
+            raise ValueError(f"rotary_halves {prefix!r}: scaling_kind {kind!r} is not supported (ramp | wavelength)")
+        if not self.dims:
+            self.freqs, self.factor = [], 1.0
+        elif kind == "wavelength":
+            self.freqs, self.factor = wavelength_scaled_frequencies(self.dims, params["base"], params.get("scaling")), 1.0
+        else:
+            self.freqs, self.factor = rescaled_frequencies(self.dims, params["base"], params.get("scaling"))
         self._device_freqs = None
 
     def bind(self, tensors):
@@ -83,20 +114,21 @@ def _pad_rows(t, multiple=16):
     return torch.cat([t, torch.zeros(extra, t.shape[1], dtype=t.dtype, device=t.device)], 0)
 
 
-def _attend(mixer, step, q, attn, kc, vc, g, nh, nkv, d, dv, scale, window):
-    """Keys and values of one size, no window, bfloat16: the kernels every attention over paged keys and values takes
-    (parts/paged_attention.py: partitioned for single rows, tiled for runs of positions).  Otherwise the window
-    attention's: steps with runs of positions take its matrix-core kernel where it has the head shape, others one
-    (row, head) per workgroup."""
+def _attend(mixer, step, q, attn, kc, vc, g, nh, nkv, d, dv, scale, window, keep_first=0, softcap=0.0):
+    """Keys and values of one size, no window, no cap on the scores, bfloat16: the kernels every attention over paged
+    keys and values takes (parts/paged_attention.py: partitioned for single rows, tiled for runs of positions).
+    Otherwise the window attention's: steps with runs of positions take its matrix-core kernel where it has the head
+    shape, others one (row, head) per workgroup."""
     ops = mixer.ctx.ops
-    if d == dv and window == 0 and attn.dtype == torch.bfloat16 and d % 8 == 0 and d <= 256:
+    if d == dv and window == 0 and not softcap and attn.dtype == torch.bfloat16 and d % 8 == 0 and d <= 256:
         return paged_attention.attend(step, ops, q, attn, kc, vc, g, nh, nkv, d, scale, 0)
     if step.max_run > 1 and ops.attention_window_pool_tiles_supported(d, dv, attn.dtype, kc.shape[2]):
         ops.attention_window_pool_tiles(q, attn, kc, vc, None, None, step.tables(g), step.table_stride(g), step.run_start,
-                                        step.seq_start, step.seqs, step.max_run, nh, nkv, d, dv, scale, window, 0)
+                                        step.seq_start, step.seqs, step.max_run, nh, nkv, d, dv, scale, window, 0,
+                                        keep_first=keep_first, softcap=softcap)
     else:
         ops.attention_window_pool(q, attn, kc, vc, None, None, step.tables(g), step.table_stride(g), step.row_seq, step.ctx_lens,
-                                  nh, nkv, d, dv, scale, window, 0, rows=step.rows)
+                                  nh, nkv, d, dv, scale, window, 0, rows=step.rows, keep_first=keep_first, softcap=softcap)
 
 
 @MIXERS.register("gated_attention")
@@ -212,3 +244,94 @@ class LatentAttention(Mixer):
         attn = step.ws("la_attn", (T, nh * r))
         _attend(self, step, q, attn, kc, vc, g, nh, 1, r, r, p["scale"], p.get("window", 0))
         return linear32(self.ctx, step, attn, w["w_o"], "la_out", keep_partial=True)
+
+
+@MIXERS.register("capped_window_attention")
+class CappedWindowAttention(Mixer):
+    """Grouped-query attention without biases.  q and k may each be divided by the root mean square over their whole
+    projection (all heads at once, before the split into heads) and multiplied by a weight of that size (``qk_norm_eps``),
+    then rotated (``position``: a PartSpec, default none).  score = (q . k) * scale, capped as softcap * tanh(score /
+    softcap) where ``softcap`` > 0; a row at position i sees j <= i with i - j < window or j < keep_first (window 0: every
+    earlier token); an ordinary softmax.  ``value_mix``: "source" keeps the values this layer's projection made at hand
+    for later layers of the step; "blend" replaces this layer's values by (1 - lambda) v + lambda v_source, v_source the
+    "source" layer's values of the same token and lambda the scalar tensor ``vmix``; the blended values are what the pages
+    hold.  params: heads, kv_heads, dim, vdim, scale, softcap, window, keep_first, qk_norm_eps, value_mix, position.
+    Tensors under the prefix: q, k, v, o, q.norm, k.norm (with qk_norm_eps), vmix (with value_mix)."""
+
+    capturable = True
+    sub_part_names = ("position",)
+
+    def __init__(self, params, prefix, ctx):
+        super().__init__(params, prefix, ctx)
+        p = params
+        self.nh, self.nkv, self.d, self.dv = p["heads"], p["kv_heads"], p["dim"], p["vdim"]
+        if self.nkv <= 0 or self.nh % self.nkv:
+            raise ValueError(f"capped_window_attention {prefix!r}: heads {self.nh} is not a multiple of kv_heads {self.nkv}")
+        self.value_mix = p.get("value_mix")
+        if self.value_mix not in (None, "source", "blend"):
+            raise ValueError(f"capped_window_attention {prefix!r}: value_mix {self.value_mix!r} is not supported (source | blend)")
+        self.window = p.get("window", 0)
+        self.keep_first = p.get("keep_first", 0) if self.window else 0
+        pos = p.get("position") or PartSpec("rotary_halves", {"dims": 0, "base": 10000.0})
+        self.position = POSITIONS.get(pos.kind)(pos.params, prefix, ctx)
+        self.mix = 0.0
+
+    def sub_parts(self):
+        return (self.position,)
+
+    def param_specs(self):
+        H, pre = self.ctx.hidden_size, self.prefix
+        sizes = (("q", self.nh * self.d), ("k", self.nkv * self.d), ("v", self.nkv * self.dv))
+        specs = [ParamSpec("w_proj", tuple((pre + n, (c, H)) for n, c in sizes)),
+                 ParamSpec("w_o", ((pre + "o", (H, self.nh * self.dv)),))]
+        if self.params.get("qk_norm_eps") is not None:
+            specs += [ParamSpec("q_norm", ((pre + "q.norm", (self.nh * self.d,)),), role="vector"),
+                      ParamSpec("k_norm", ((pre + "k.norm", (self.nkv * self.d,)),), role="vector")]
+        if self.value_mix == "blend":
+            specs.append(ParamSpec("mix", ((pre + "vmix", ()),), role="vector"))
+        return specs
+
+    def ignorable_tensors(self):
+        return () if self.value_mix == "blend" else (self.prefix + "vmix",)      # a layer that does not blend may still carry one
+
+    def bind(self, tensors):
+        small = f32_params({k: tensors[k] for k in ("q_norm", "k_norm") if k in tensors})
+        if "mix" in tensors:      # a constant of the model: read once, handed to the kernel as a number
+            self.mix = float(tensors["mix"].float().reshape(-1)[0].item())
+        super().bind({"w_proj": _pad_rows(tensors["w_proj"]), "w_o": tensors["w_o"], **small})
+
+    def cache_need(self):
+        return KVCacheNeed(self.nkv, self.d, self.window, value_dim=self.dv, keep_first=self.keep_first)
+
+    def flops(self, rows, attended=0):
+        seen = min(attended, rows * (self.window + self.keep_first)) if self.window else attended
+        return super().flops(rows) + 2.0 * seen * (self.d + self.dv) * self.nh
+
+    def forward(self, step, h):
+        ops, p, w = self.ctx.ops, self.params, self.w
+        g = self.cache.group
+        kc, vc = self.cache.k(self.cache_index), self.cache.v(self.cache_index)
+        T = step.rows
+        proj = linear32(self.ctx, step, h, w["w_proj"], "cwa_proj")
+        q = step.ws("cwa_q", (T, self.nh * self.d))
+        slots = step.slots(g) if self.cache_owner else None
+        source = None
+        if self.value_mix is not None:      # the step's rows of values that the "source" layer made, one buffer per size
+            key = ("value_mix_source", self.nkv * self.dv)
+            if self.value_mix == "source":
+                source = step.shared[key] = step.ws("values_of_source", (T, self.nkv * self.dv), torch.float32)
+            else:
+                source = step.shared.get(key)
+                if source is None:
+                    raise RuntimeError(f"capped_window_attention {self.prefix!r} blends its values with a layer's that has not run "
+                                       "(value_mix 'source' must come first)")
+        ops.norm_rotate_store(proj, q, self.nh, self.nkv, self.d, self.dv, p.get("qk_norm_eps") or 0.0,
+                              q_weight=w.get("q_norm"), k_weight=w.get("k_norm"),
+                              v_other=source if self.value_mix == "blend" else None, mix=self.mix,
+                              v_keep=source if self.value_mix == "source" else None,
+                              cos_sin=self.position.pairs_table(step), rot=self.position.params["dims"], slots=slots,
+                              kcache=kc, vcache=vc, rows=T, halves=True)
+        attn = step.ws("cwa_attn", (T, self.nh * self.dv))
+        _attend(self, step, q, attn, kc, vc, g, self.nh, self.nkv, self.d, self.dv, p["scale"], self.window,
+                keep_first=self.keep_first, softcap=float(p.get("softcap") or 0.0))
+        return linear32(self.ctx, step, attn, w["w_o"], "cwa_out", keep_partial=True)      # the stream's next norm adds the slices

@@ -244,7 +244,8 @@ class TokenEmbedding(Embedding):
 class LinearHead(Head):
     """logits = h @ table^T in 32-bit, only for the rows that are asked for
     (src/model/llama.cpp:126-128).  params: vocab_size, tied (use the embedding's table), scale (a factor on the
-    logits, default 1: applied to the 32-bit logits)."""
+    logits, default 1: applied to the 32-bit logits), softcap (c > 0: logits <- c tanh(logits / c) after the factor;
+    default none)."""
 
     capturable = True
 
@@ -264,6 +265,8 @@ class LinearHead(Head):
         self.ctx.ops.gemm(h, self.w["table"], out, tuning=step.tune_products)
         if float(self.params.get("scale", 1.0)) != 1.0:
             self.ctx.ops.scale_rows(out, self.params["scale"])
+        if float(self.params.get("softcap") or 0.0) > 0.0:
+            self.ctx.ops.softcap_rows(out, self.params["softcap"])
         return out
 
 
