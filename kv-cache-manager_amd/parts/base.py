@@ -59,10 +59,13 @@ class ParamSpec:
     dim 0 in that order (one pair = taken as it is).  ``role`` decides the stored precision:
       matrix / table  the compute dtype (bfloat16 when serving, float32 in the 32-bit path)
       vector          as stored when that is 32-bit, else the compute dtype
-      index           integer tables, kept as int32."""
+      index           integer tables, kept as int32.
+    ``distinct_below`` (index tables): what valid entries look like, for whoever makes random ones: every row holds
+    distinct values in [0, distinct_below) (0: any values)."""
     name: str
     sources: Tuple[Tuple[str, Tuple[int, ...]], ...]
     role: str = "matrix"
+    distinct_below: int = 0
 
     @property
     def shape(self):

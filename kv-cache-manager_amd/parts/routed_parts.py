@@ -61,7 +61,7 @@ class RoutedExperts(FeedForward):
         if self.gated:
             specs.append(ParamSpec("w_gate", tuple((n + p.get("gate", "gate"), (F, H)) for n in names)))
         if self.routing == "table":
-            specs.append(ParamSpec("table", ((pre + p.get("table", "table"), (p.get("vocab_size", -1), p["top"])),), role="index"))
+            specs.append(ParamSpec("table", ((pre + p.get("table", "table"), (p.get("vocab_size", -1), p["top"])),), role="index", distinct_below=E))
         else:
             specs.append(ParamSpec("w_router", ((pre + p.get("router", "router"), (E, H)),)))
         return specs

@@ -76,9 +76,18 @@ def index_values(key: int, count: int, modulus: int = INDEX_MODULUS) -> np.ndarr
     return (_counters(key, 0, count) % np.uint64(modulus)).astype(np.int32)
 
 
-def random_tensor(seed: int, name: str, shape, role: str, dtype=torch.bfloat16, std=0.02, norm_jitter=0.0, device="cpu"):
-    """One tensor of the rule.  role "vector": 1 + norm_jitter * n; "index": int32 in [0, INDEX_MODULUS);
-    else std * n.  On a GPU the fill kernel makes the values in place."""
+def _distinct_rows(raw: torch.Tensor, below: int) -> torch.Tensor:
+    """An index table whose rows hold distinct values in [0, below): a row's first raw value, and its successors."""
+    if raw.dim() != 2 or raw.shape[1] > below:
+        raise ValueError(f"a table of {tuple(raw.shape)} cannot hold distinct values below {below} in every row")
+    step = torch.arange(raw.shape[1], dtype=torch.int32, device=raw.device)
+    return ((raw[:, :1] + step) % below).to(torch.int32).contiguous()
+
+
+def random_tensor(seed: int, name: str, shape, role: str, dtype=torch.bfloat16, std=0.02, norm_jitter=0.0, device="cpu",
+                  distinct_below=0):
+    """One tensor of the rule.  role "vector": 1 + norm_jitter * n; "index": int32 in [0, INDEX_MODULUS), or with
+    ``distinct_below`` rows of distinct values below that; else std * n.  On a GPU the fill kernel makes the values in place."""
     if any(n < 0 for n in shape):
         raise ValueError(f"{name}: a size of this tensor is left to the checkpoint ({tuple(shape)}); random weights need it in "
                          "the configuration")
@@ -89,6 +98,8 @@ def random_tensor(seed: int, name: str, shape, role: str, dtype=torch.bfloat16, 
     if dev.type == "cuda":
         from .. import ops
         if role == "index":
+            if distinct_below:
+                return _distinct_rows(ops.fill_index(torch.empty(shape, dtype=torch.int32, device=dev), key, 1 << 20), distinct_below)
             return ops.fill_index(torch.empty(shape, dtype=torch.int32, device=dev), key, INDEX_MODULUS)
         store = dtype if dtype in (torch.float32, torch.bfloat16) else torch.float32
         t = torch.empty(shape, dtype=store, device=dev)
@@ -98,6 +109,8 @@ def random_tensor(seed: int, name: str, shape, role: str, dtype=torch.bfloat16, 
             ops.fill_normal(t, key, mean, scale)
         return t.to(dtype)
     if role == "index":
+        if distinct_below:
+            return _distinct_rows(torch.from_numpy(index_values(key, count, 1 << 20).reshape(shape)), distinct_below)
         return torch.from_numpy(index_values(key, count).reshape(shape))
     if scale == 0.0:
         return torch.full(shape, mean, dtype=torch.float32).to(dtype)
@@ -118,9 +131,19 @@ def expected_tensors(architecture: str, config) -> Dict[str, tuple]:
     return out
 
 
+def index_rules(architecture: str, config) -> Dict[str, int]:
+    """Checkpoint names of the index tables whose rows must hold distinct values below a bound -> that bound."""
+    arch = ARCHITECTURES.get(architecture)
+    spec = arch.build_spec(config)
+    model = Model(spec, BuildContext(torch.float32, torch.device("cpu"), spec.hidden_size, 16, None))
+    return {name: ps.distinct_below for part in model.every_part() for ps in part.param_specs() if ps.distinct_below
+            for name, _ in ps.sources}
+
+
 def random_tensors(architecture: str, config, seed: int, dtype=torch.bfloat16, std=0.02, norm_jitter=0.0,
                    device="cpu") -> Dict[str, torch.Tensor]:
-    return {name: random_tensor(seed, name, shape, role, dtype, std, norm_jitter, device)
+    rules = index_rules(architecture, config)
+    return {name: random_tensor(seed, name, shape, role, dtype, std, norm_jitter, device, distinct_below=rules.get(name, 0))
             for name, (shape, role) in expected_tensors(architecture, config).items()}
 
 
