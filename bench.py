@@ -3,7 +3,7 @@
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512] [--layers L]
                   [--sizes tinyllama-1.1b|llama-2-7b|llama-3-8b] [--context-limit 2048] [--prefill-tokens 2048]
                   [--tune-products off|heuristic|all] [--no-points] [--only-prefill]
-  python bench.py --design kasuvik|furapel [--design-sizes 2048,4096] [--layers 4] [--prefill-tokens 2048] [--steps K]
+  python bench.py --design kasuvik|furapel|fisesun [--design-sizes 2048,4096] [--layers 4] [--prefill-tokens 2048] [--steps K]
 
 A "step" is one decode step of the whole engine (schedule, batch metadata, upload, model step on
 the GPU, sampling, download, update).  W untimed steps, then exactly K timed steps between two
@@ -18,6 +18,10 @@ depth, both with random weights through the same engine.  One JSON line with bot
 --design furapel does the same for the Furapel decoder (side-by-side layers with dynamic tanh norms: gated grouped-query
 attention, latent attention over a window, a matrix memory with exponential gates, routed experts) beside the Kasuvik
 and the Llama decoder at equal width, heads, active feed-forward width and depth.
+
+--design fisesun does the same for the Fisesun decoder (layers that norm a sublayer's output only: grouped-query attention
+with q and k normed over the whole projection, capped scores, a window that keeps the first tokens, blended values; a
+matrix memory; gated experts named by a table per token id beside a shared expert) beside the Furapel and the Llama decoder.
 """
 import argparse
 import json
@@ -189,6 +193,29 @@ def furapel_config(width, layers, vocab=32000):
                                     "loop": {"start": 0, "stop": 1, "times": 1}})
 
 
+# Fisesun at a width: (first tokens a window keeps, cap on the scores, experts, experts a row); the other sizes are DESIGN_SIZES'
+FISESUN_SIZES = {2048: (4, 50.0, 8, 2), 4096: (4, 50.0, 8, 2)}
+
+
+def fisesun_config(width, layers, vocab=32000):
+    """A Fisesun configuration at a width of DESIGN_SIZES: layers attention, attention, matrix memory, attention in turn
+    (the attention layers blend their values with the first one's), each followed by ``experts`` gated experts of which a
+    row uses ``top`` and a shared expert (the ``top`` experts a quarter each and the shared one half of the dense
+    feed-forward's width)."""
+    from kvcm_amd.config.fisesun_config import FisesunConfig
+    nh, nkv, hd, ff, window = DESIGN_SIZES[width][:5]
+    keep, cap, experts, top = FISESUN_SIZES[width]
+    mlp = {"kind": "moe", "expert": {"ff": ff // (2 * top)}, "router": {"experts": experts, "top": top}, "shared": {"ff": ff // 2}}
+    attention = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": cap, "v_mix": True,
+                 "mask": {"size": window, "keep_first": keep},
+                 "rot": {"dims": hd, "base": 500000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    memory = {"heads": nh, "dim": hd, "vdim": hd, "gate_cap": 15.0}
+    kinds = [("attention", attention), ("attention", attention), ("mlstm", memory), ("attention", attention)]
+    listed = [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": mlp} for i in range(layers)]
+    return FisesunConfig.from_dict({"architecture": "Fisesun", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+                                    "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "layers": listed})
+
+
 def design_main(args):
     import torch
     from kvcm_amd.config.engine_config import EngineConfig
@@ -202,7 +229,8 @@ def design_main(args):
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
     first = args.design
     record = {"metric": "prefill and decode tok/s of the %s decoder beside the %s at equal sizes"
-                        % (first.capitalize(), "Llama decoder" if first == "kasuvik" else "Kasuvik and Llama decoders"), "dtype": key,
+                        % (first.capitalize(), {"kasuvik": "Llama decoder", "furapel": "Kasuvik and Llama decoders",
+                                                 "fisesun": "Furapel and Llama decoders"}[first]), "dtype": key,
               "data": "synthetic", "layers": layers, "prefill_tokens": T, "prompt_len": args.prompt_len, "steps": steps, "sizes": {}}
     for width in [int(w) for w in args.design_sizes.split(",")]:
         if width not in DESIGN_SIZES:
@@ -212,8 +240,12 @@ def design_main(args):
         designs = dict(zip(("kasuvik", "llama"), kasuvik_pair(width, layers)))
         if first == "furapel":
             designs = {"furapel": furapel_config(width, layers), **designs}
+        elif first == "fisesun":
+            designs = {"fisesun": fisesun_config(width, layers), "furapel": furapel_config(width, layers), "llama": designs["llama"]}
+        if args.design_alone:
+            designs = {first: designs[first]}
         for name, cfg in designs.items():
-            arch = {"kasuvik": "Kasuvik", "furapel": "Furapel", "llama": "LlamaForCausalLM"}[name]
+            arch = {"kasuvik": "Kasuvik", "furapel": "Furapel", "fisesun": "Fisesun", "llama": "LlamaForCausalLM"}[name]
             tensors = random_tensors(arch, cfg, seed=0, dtype=dt, device="cuda:0")
             ec = EngineConfig(block_size=16, max_seq_len=limit, num_blocks=8 * limit // 16, max_num_seqs=8,
                               max_batched_tokens=max(4096, T + 64), dtype=args.dtype, max_logit_rows=64, beyond_max_position=True)
@@ -234,6 +266,9 @@ def design_main(args):
             entry[name] = one
             del eng
             torch.cuda.empty_cache()
+        if args.design_alone:
+            record["sizes"][str(width)] = entry
+            continue
         entry["prefill_ratio"] = round(entry[first]["prefill_tok_s"] / entry["llama"]["prefill_tok_s"], 3)
         entry["decode_b8_ratio"] = round(entry[first]["decode_b8_tok_s"] / entry["llama"]["decode_b8_tok_s"], 3)
         record["sizes"][str(width)] = entry
@@ -263,11 +298,13 @@ def main():
                     help="run nothing but the 2,048-token prefill (for a profiler); prints its record alone")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="tokens of the prefill measurement (2,048 in the record; other lengths for sweeps)")
-    ap.add_argument("--design", default="llama", choices=["llama", "kasuvik", "furapel"],
+    ap.add_argument("--design", default="llama", choices=["llama", "kasuvik", "furapel", "fisesun"],
                     help="llama: the workload above (the default); kasuvik: prefill and decode of the Kasuvik decoder beside the "
-                         "Llama decoder at equal sizes; furapel: the same for the Furapel decoder beside both "
+                         "Llama decoder at equal sizes; furapel: the same for the Furapel decoder beside both; "
+                         "fisesun: the same for the Fisesun decoder beside the Furapel and the Llama decoder "
                          "(--design-sizes, --layers, --prefill-tokens, --prompt-len, --steps)")
     ap.add_argument("--design-sizes", default="2048,4096", help="widths of the --design comparison (2048, 4096)")
+    ap.add_argument("--design-alone", action="store_true", help="run the --design itself only, not the designs beside it (for a profiler)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus N with N > 1 is not supported")
