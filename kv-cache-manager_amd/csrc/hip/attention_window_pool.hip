@@ -91,6 +91,11 @@ __global__ void __launch_bounds__(256)
 // of that size (wq, wk; null: that stretch passes as it is).  v may be blended with the values another layer made for the
 // same row, v <- (1 - mix) v + mix * v_other (v_other null: none); v_keep (null: none) receives the row's values as the
 // projection made them, for later layers to blend with.  What is stored in the pages is the blended v.
+// Grid (rows, parts).  parts 1: one workgroup does a whole row.  parts nh + nkv + 1, for steps of few rows: workgroup y
+// does head y of q | k (it sums the squares of that head's whole stretch itself, in the same order, so the bits are those
+// of the one-workgroup form) and the last one the values.
+constexpr int kNormRotateFewRows = 16;
+
 template <class T>
 __global__ void __launch_bounds__(256)
     norm_rotate_store_kernel(const float* __restrict__ src, int ld, const float* __restrict__ wq, const float* __restrict__ wk,
@@ -102,13 +107,21 @@ __global__ void __launch_bounds__(256)
   const int row = blockIdx.x;
   const float* r = src + size_t(row) * ld;
   const int nq = nh * d, nk = nkv * d;
+  int e0 = 0, e1 = nq + nk;
+  bool values = true;
+  if (gridDim.y > 1) {
+    const int part = blockIdx.y;
+    values = part == nh + nkv;
+    e0 = values ? 0 : part * d;
+    e1 = values ? 0 : e0 + d;
+  }
   float inv_q = 1.f, inv_k = 1.f;
-  if (wq) {
+  if (wq && e0 < nq && e1 > e0) {
     float ss = 0.f;
     for (int e = threadIdx.x; e < nq; e += 256) ss = fmaf(r[e], r[e], ss);
     inv_q = 1.0f / sqrtf(block_sum<256>(ss, scratch) / float(nq) + eps);
   }
-  if (wk) {
+  if (wk && e1 > nq) {
     float ss = 0.f;
     for (int e = threadIdx.x; e < nk; e += 256) ss = fmaf(r[nq + e], r[nq + e], ss);
     inv_k = 1.0f / sqrtf(block_sum<256>(ss, scratch) / float(nk) + eps);
@@ -120,7 +133,7 @@ __global__ void __launch_bounds__(256)
   };
   const float2* cs = cos_sin + size_t(row) * (rot / 2);
   const int slot = slots ? slots[row] : -1;
-  for (int e = threadIdx.x; e < nq + nk; e += 256) {
+  for (int e = e0 + threadIdx.x; e < e1; e += 256) {
     const int head = e / d, i = e % d;
     float x = normed(e);
     if (i < rot) {
@@ -133,6 +146,7 @@ __global__ void __launch_bounds__(256)
     if (head < nh) store_f(q_out + size_t(row) * ldq + e, x);
     else if (slot >= 0) store_f(kcache + ((size_t(slot / B) * nkv + (head - nh)) * B + slot % B) * d + i, x);
   }
+  if (!values) return;
   const float* v = r + nq + nk;
   for (int e = threadIdx.x; e < nkv * dv; e += 256) {
     float x = v[e];
@@ -451,12 +465,14 @@ int kvcm_norm_rotate_store(const float* src, int ld, const float* wq, const floa
   KVCM_REQUIRE((!v_other || ldvo >= nkv * dv) && (!v_keep || ldvk >= nkv * dv), "norm_rotate_store: rows of values too short");
   KVCM_REQUIRE(!slots || (kcache && vcache), "norm_rotate_store: slots without pages");
   const float2* cs = reinterpret_cast<const float2*>(cos_sin);
+  // few rows: a workgroup per head, so that a single row is not the work of one compute unit (the same bits either way)
+  const dim3 grid(T, T <= kNormRotateFewRows ? nh + nkv + 1 : 1);
   if (dtype == kF32)
-    norm_rotate_store_kernel<float><<<T, 256, 0, s>>>(src, ld, wq, wk, eps, v_other, ldvo, mix, v_keep, ldvk, cs, rot, halves, slots,
+    norm_rotate_store_kernel<float><<<grid, 256, 0, s>>>(src, ld, wq, wk, eps, v_other, ldvo, mix, v_keep, ldvk, cs, rot, halves, slots,
                                                        static_cast<float*>(q_out), ldq, static_cast<float*>(kcache),
                                                        static_cast<float*>(vcache), nh, nkv, d, dv, B);
   else if (dtype == kBF16)
-    norm_rotate_store_kernel<bf16_t><<<T, 256, 0, s>>>(src, ld, wq, wk, eps, v_other, ldvo, mix, v_keep, ldvk, cs, rot, halves, slots,
+    norm_rotate_store_kernel<bf16_t><<<grid, 256, 0, s>>>(src, ld, wq, wk, eps, v_other, ldvo, mix, v_keep, ldvk, cs, rot, halves, slots,
                                                         static_cast<bf16_t*>(q_out), ldq, static_cast<bf16_t*>(kcache),
                                                         static_cast<bf16_t*>(vcache), nh, nkv, d, dv, B);
   else KVCM_REQUIRE(false, "norm_rotate_store: unknown dtype %d", dtype);

@@ -90,11 +90,13 @@ __global__ void __launch_bounds__(kChainThreads)
 
 // The same chain for rows whose length is a multiple of 4 and at most 1024 * G (G groups of four values a thread):
 // the branches' and the stream's values of a row are read once, 16 bytes a load, and stay in registers through all
-// stages, so the row costs one trip to memory instead of one per stage.  Which of the two kernels runs depends on the
-// row length (and on whether a branch is still in slices) only, never on the batch.
+// stages, so the row costs one trip to memory instead of one per stage.  A branch that is still the slices of a split
+// product is added up as it is read, slice after slice.  Which of the two kernels runs depends on the row length only,
+// never on the batch.
 template <class TO, int G>
 __global__ void __launch_bounds__(kChainThreads)
-    rmsnorm_chain_rows_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
+    rmsnorm_chain_rows_kernel(float* __restrict__ x, const float* __restrict__ a, int a_splits, const float* __restrict__ b,
+                              int b_splits, size_t split_stride,
                               const float* __restrict__ wa, const float* __restrict__ wb, float combine,
                               const float* __restrict__ w_post, const int* __restrict__ rows,
                               const float* __restrict__ w_pre, TO* __restrict__ out, int H, float eps, int write_back) {
@@ -113,11 +115,23 @@ __global__ void __launch_bounds__(kChainThreads)
     const float4 vx = *reinterpret_cast<const float4*>(xr + ic);
     xv[g][0] = vx.x; xv[g][1] = vx.y; xv[g][2] = vx.z; xv[g][3] = vx.w;
     if (a) {
-      const float4 va = *reinterpret_cast<const float4*>(a + size_t(src) * H + ic);
+      const float* p = a + size_t(src) * H + ic;
+      float4 va = *reinterpret_cast<const float4*>(p);
+#pragma unroll 4
+      for (int sl = 1; sl < a_splits; ++sl) {
+        const float4 t = *reinterpret_cast<const float4*>(p + size_t(sl) * split_stride);
+        va.x += t.x; va.y += t.y; va.z += t.z; va.w += t.w;
+      }
       av[g][0] = va.x; av[g][1] = va.y; av[g][2] = va.z; av[g][3] = va.w;
     }
     if (b) {
-      const float4 vb = *reinterpret_cast<const float4*>(b + size_t(src) * H + ic);
+      const float* p = b + size_t(src) * H + ic;
+      float4 vb = *reinterpret_cast<const float4*>(p);
+#pragma unroll 4
+      for (int sl = 1; sl < b_splits; ++sl) {
+        const float4 t = *reinterpret_cast<const float4*>(p + size_t(sl) * split_stride);
+        vb.x += t.x; vb.y += t.y; vb.z += t.z; vb.w += t.w;
+      }
       bv[g][0] = vb.x; bv[g][1] = vb.y; bv[g][2] = vb.z; bv[g][3] = vb.w;
     }
   }
@@ -227,10 +241,11 @@ int kvcm_rmsnorm_chain(float* x, const float* a, int a_splits, const float* b, i
   KVCM_REQUIRE(!out || out_dtype == kF32 || out_dtype == kBF16, "rmsnorm_chain: unknown output dtype %d", out_dtype);
   const bool f32 = !out || out_dtype == kF32;
   auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  if (a_splits == 1 && b_splits == 1 && H % 4 == 0 && H <= 8192 && aligned(x) && aligned(a) && aligned(b)) {
+  if (H % 4 == 0 && H <= 8192 && aligned(x) && aligned(a) && aligned(b)) {      // slices lie split_stride = T * H floats apart
 #define KVCM_CHAIN_ROWS(TO, G)                                                                                     \
-  rmsnorm_chain_rows_kernel<TO, G><<<R, kChainThreads, 0, s>>>(x, a, b, wa, wb, combine, w_post, rows, w_pre,      \
-                                                               static_cast<TO*>(out), H, eps, wb_flag)
+  rmsnorm_chain_rows_kernel<TO, G><<<R, kChainThreads, 0, s>>>(x, a, a_splits, b, b_splits,                         \
+                                                               static_cast<size_t>(split_stride), wa, wb, combine, \
+                                                               w_post, rows, w_pre, static_cast<TO*>(out), H, eps, wb_flag)
     if (H <= 2048) { if (f32) KVCM_CHAIN_ROWS(float, 2); else KVCM_CHAIN_ROWS(bf16_t, 2); }
     else if (H <= 4096) { if (f32) KVCM_CHAIN_ROWS(float, 4); else KVCM_CHAIN_ROWS(bf16_t, 4); }
     else { if (f32) KVCM_CHAIN_ROWS(float, 8); else KVCM_CHAIN_ROWS(bf16_t, 8); }
