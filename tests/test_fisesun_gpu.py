@@ -61,10 +61,12 @@ def test_the_stream_read_as_it_is_and_capped_logits():
             ops.rmsnorm_chain(dev(x), 1e-5, out=out2, plain=True)
             np.testing.assert_allclose(out2.float().cpu().numpy(), x, atol=tol * np.abs(x).max())
         # the output still to be added as the slices of a split product
-        sl = rng.normal(size=(3, T, H))
-        xs, out = dev(x), torch.empty(T, H, device=DEV)
-        ops.rmsnorm_chain(xs, 1e-5, pending=ops.NormedBranches(ops.PartialSums(dev(sl), 3, T, H, torch.empty(T, H, device=DEV)), dev(w)), out=out, plain=True)
-        np.testing.assert_allclose(out.cpu().numpy(), x + plain.rms(sl.sum(0), 1e-5) * w, atol=5e-6)
+        for S in (3, 9):
+            sl = rng.normal(size=(S, T, H))
+            xs, out = dev(x), torch.empty(T, H, device=DEV)
+            ops.rmsnorm_chain(xs, 1e-5, pending=ops.NormedBranches(ops.PartialSums(dev(sl), S, T, H, torch.empty(T, H, device=DEV)), dev(w)), out=out, plain=True)
+            np.testing.assert_allclose(out.cpu().numpy(), x + plain.rms(sl.sum(0), 1e-5) * w, atol=5e-6)
+            np.testing.assert_allclose(xs.cpu().numpy(), out.cpu().numpy(), atol=0)      # the stream holds what its reader got
     z = rng.normal(size=(4, 77)) * 20
     zs = dev(z)
     ops.softcap_rows(zs, 7.5)
@@ -116,6 +118,15 @@ def test_projection_normed_over_all_heads_rotated_blended_and_stored(case):
             if s >= 0:
                 np.testing.assert_allclose(kc[s // B, :, s % B].cpu().numpy(), want_k[t], atol=1e-5)
                 np.testing.assert_allclose(vc[s // B, :, :, s % B].cpu().numpy(), v_ref[t].reshape(nkv, dv), atol=2e-6)
+    # steps of few rows take a workgroup per head, steps of many one per row: the same bits
+    many = 5
+    big, slots_big = dev(np.tile(proj, (many, 1))), torch.cat([slots] + [torch.full_like(slots, -1)] * (many - 1))
+    table_big = table.repeat(many, 1) if rot else None
+    q_big = torch.empty(many * T, nh * d, device=DEV)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ops.norm_rotate_store(big, q_big, nh, nkv, d, dv, eps, q_weight=dev(w["q.norm"]), k_weight=dev(w["k.norm"]), cos_sin=table_big, rot=rot,
+                          slots=slots_big, kcache=kc2, vcache=vc2, halves=True)
+    assert torch.equal(q_big[:T], q_out) and torch.equal(q_big[-T:], q_out) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
     # without weights the projection passes as rotate_store leaves it
     q_a, q_b = torch.empty(T, nh * d, device=DEV), torch.empty(T, nh * d, device=DEV)
     ops.norm_rotate_store(dev(proj), q_a, nh, nkv, d, dv, 0.0, cos_sin=table, rot=rot, halves=True)
