@@ -67,8 +67,9 @@ __global__ void __launch_bounds__(256)
     moe_grouped_kernel(const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, const int* __restrict__ order,
                        const int* __restrict__ tiles, int top, void* __restrict__ out, const float* __restrict__ weight, int N,
                        int K, int col_blocks) {
-  __shared__ __attribute__((aligned(16))) uint16_t As[kGM][kGPitch];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[kGN][kGPitch];
+  __shared__ __attribute__((aligned(16))) uint16_t staged[2][kGM][kGPitch];      // both operands; the down form's results pass through it too
+  uint16_t (*As)[kGPitch] = staged[0];
+  uint16_t (*Bs)[kGPitch] = staged[1];
   __shared__ int pair_of[kGM];
   // The chip hands consecutive workgroups to its eight XCDs in turn, each with an L2 of its own.  Workgroup L goes to
   // XCD L % 8; it takes a column block that is congruent to its XCD and walks the tiles in order, so that the tiles of
@@ -140,6 +141,44 @@ __global__ void __launch_bounds__(256)
     __syncthreads();
   }
   // accumulator layout: a lane holds column lane % 16 and rows 4 * (lane / 16) + r of each 16 x 16 tile
+  if constexpr (MODE == kDown) {
+    // 32-bit results by pair: stored from the accumulators a wave's store would write 64-byte pieces of four rows.  Each
+    // wave passes its 64 x 64 results through LDS instead, 32 rows at a time, and writes whole 256-byte stretches of
+    // a row, 16 bytes a lane.  The operands' space is free by now (the loop ended with a barrier).
+    constexpr int kPitch = 68;      // floats; 4 waves x 32 rows x 68 fit the operands' 9,216 floats
+    static_assert(4 * 32 * kPitch * sizeof(float) <= sizeof(staged), "the results of half a tile must fit the operands' space");
+    float* mine = reinterpret_cast<float*>(&staged[0][0][0]) + wave * 32 * kPitch;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            mine[(ii * 16 + (lane / 16) * 4 + r) * kPitch + j * 16 + lane % 16] = acc[half * 2 + ii][j][r];
+      __syncthreads();
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int idx = it * kWave + lane, rl = idx / 16, c4 = (idx % 16) * 4;
+        const int m = wm * 64 + half * 32 + rl;
+        const int c = n0 + wn * 64 + c4;
+        if (m >= rows || c >= N) continue;
+        const int pair = pair_of[m];
+        const float g = weight[pair];
+        const float4 v = *reinterpret_cast<const float4*>(mine + rl * kPitch + c4);
+        float* dst = static_cast<float*>(out) + static_cast<long long>(pair) * N + c;
+        if (c + 3 < N && N % 4 == 0) {
+          *reinterpret_cast<float4*>(dst) = float4{g * v.x, g * v.y, g * v.z, g * v.w};
+        } else {
+          const float e4[4] = {v.x, v.y, v.z, v.w};
+          for (int q = 0; q < 4 && c + q < N; ++q) dst[q] = g * e4[q];
+        }
+      }
+      __syncthreads();
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
