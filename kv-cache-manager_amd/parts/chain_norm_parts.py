@@ -147,7 +147,7 @@ class ScaledTokenEmbedding(Embedding):
 @FEED_FORWARDS.register("gated_mlp")
 class GatedFeedForward(FeedForward):
     """down(act(gate(h)) * up(h)), gate and up as one fused projection whose 32-bit sums go straight into the
-    activation.  params: intermediate_size, activation ("relu" | "silu" | "gelu_tanh"); gate, up, down: the
+    activation (steps of few rows in bfloat16 with silu: in the product's own epilogue).  params: intermediate_size, activation ("relu" | "silu" | "gelu_tanh"); gate, up, down: the
     checkpoint names after the prefix (defaults "gate", "up", "down").  The result is 32-bit: a norm reads it."""
 
     capturable = True
@@ -159,7 +159,11 @@ class GatedFeedForward(FeedForward):
 
     def forward(self, step, h):
         I, ops = self.params["intermediate_size"], self.ctx.ops
-        gu = linear32(self.ctx, step, h, self.w["w_gate_up"], "gated_gate_up")
         act = step.ws("gated_act", (step.rows, I))
-        ops.gated_act(gu, act, self.params.get("activation", "silu"))
+        kind = self.params.get("activation", "silu")
+        # few rows in bfloat16 with silu: the product that streams gate and up rows together and applies the activation
+        # in its epilogue, one launch (the activation is rounded once more on the way, within the result's own rounding)
+        if not (kind == "silu" and act.dtype == torch.bfloat16 and torch.is_tensor(h) and ops.gemm_swiglu(h, self.w["w_gate_up"], act)):
+            gu = linear32(self.ctx, step, h, self.w["w_gate_up"], "gated_gate_up")
+            ops.gated_act(gu, act, kind)
         return linear32(self.ctx, step, act, self.w["w_down"], "gated_out")
