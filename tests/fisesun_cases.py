@@ -51,12 +51,12 @@ CONFIGS = {
                      _layer(_attention(4, 2, 16, 24, 0.3, cap=5.0, window=20, keep=3, rot=8, base=100.0, scaling=(3.0, 1.0, 4.0, 40), v_mix=True), _moe(5, 3, 20, shared=24)),
                      _layer(_attention(2, 2, 12, 24, 0.25, cap=50.0, rot=12, base=50.0, v_mix=True), _dense(40)),
                      _layer(_attention(6, 2, 8, 24, 0.4, window=7, keep=0, v_mix=True), _moe(3, 1, 7))]},
-    # head shapes of the matrix-core kernels (keys 64, values 48 and 64), a rotation of the whole head with rescaling that
+    # head shapes of the matrix-core kernels (keys 64, values 40 and 64), a rotation of the whole head with rescaling that
     # touches every band, more kept tokens than a page holds and more than the window, a window longer than a page
     "Q": {"architecture": "Fisesun", "vocab": 130, "width": 64, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
-          "layers": [_layer(_attention(2, 1, 64, 48, 0.11, cap=20.0, window=33, keep=21, rot=64, base=5000.0, scaling=(8.0, 1.0, 4.0, 256), v_mix=True), _moe(4, 2, 32, shared=16)),
+          "layers": [_layer(_attention(2, 1, 64, 40, 0.11, cap=20.0, window=33, keep=21, rot=64, base=5000.0, scaling=(8.0, 1.0, 4.0, 256), v_mix=True), _moe(4, 2, 32, shared=16)),
                      _layer(_memory(2, 32, 16, 8.0), _moe(6, 2, 16)),
-                     _layer(_attention(4, 1, 64, 48, 0.13, cap=20.0, window=10, keep=40, rot=32, base=300.0, v_mix=True), _dense(96)),
+                     _layer(_attention(4, 1, 64, 40, 0.13, cap=20.0, window=10, keep=40, rot=32, base=300.0, v_mix=True), _dense(96)),
                      _layer(_attention(2, 2, 32, 64, 0.2, window=40, keep=5), _moe(2, 2, 48, shared=32))]},
     # one head, one expert, as many experts a token as there are, no rotation, no cap anywhere, no logit cap and no
     # embedding factor in the file, a single blending layer (nobody to blend with), a window of one token that keeps two

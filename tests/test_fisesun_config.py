@@ -64,7 +64,7 @@ def test_parts_cache_groups_and_tensors_of_a_configuration():
     model = Model(spec, BuildContext(torch.bfloat16, torch.device("cpu"), spec.hidden_size, 16, None))
     assert model.capturable, model.not_capturable()
     needs = [g.need for g in model.groups]
-    assert KVCacheNeed(1, 64, 33, value_dim=48, keep_first=21) in needs and KVCacheNeed(1, 64, 10, value_dim=48, keep_first=40) in needs
+    assert KVCacheNeed(1, 64, 33, value_dim=40, keep_first=21) in needs and KVCacheNeed(1, 64, 10, value_dim=40, keep_first=40) in needs
     assert KVCacheNeed(2, 32, 40, value_dim=64, keep_first=5) in needs and StateNeed((2, 32, 16), torch.float32) in needs
     groups = plan_groups(model, 50, 4)
     windows = sorted((g.window, g.keep_first) for g in groups if g.kind == "window")
@@ -139,7 +139,7 @@ def test_plain_frequencies_by_wavelength():
         s = (50 * f[i] / (2 * np.pi) - 2.0) / 3.0
         assert 0 < s < 1 and abs(g[i] - ((1 - s) * f[i] / 4 + s * f[i])) < 1e-15
     from kvcm_amd.parts.gated_attention_parts import wavelength_scaled_frequencies
-    for dims, base, sc in ((8, 10.0, (4.0, 2.0, 5.0, 50)), (64, 1e6, (8.0, 1.0, 4.0, 2048)), (2, 3.0, None), (32, 500.0, (2.0, 0.5, 64.0, 100))):
+    for dims, base, sc in ((8, 10.0, (4.0, 2.0, 5.0, 50)), (64, 5e5, (8.0, 1.0, 4.0, 8192)), (2, 3.0, None), (32, 500.0, (2.0, 0.5, 64.0, 100))):
         np.testing.assert_allclose(wavelength_scaled_frequencies(dims, base, sc),
                                    plain.pair_frequencies(dims, base, dict(zip(("factor", "low", "high", "original"), sc)) if sc else None), rtol=1e-13)
 

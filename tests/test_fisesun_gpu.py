@@ -74,7 +74,7 @@ def test_the_stream_read_as_it_is_and_capped_logits():
 
 
 @pytest.mark.parametrize("case", [dict(nh=3, nkv=1, d=16, dv=6, rot=8, base=100.0, sc=(3.0, 1.0, 4.0, 40)),
-                                  dict(nh=4, nkv=2, d=64, dv=48, rot=64, base=1e6, sc=(8.0, 1.0, 4.0, 2048)),
+                                  dict(nh=6, nkv=2, d=64, dv=40, rot=64, base=5e5, sc=(8.0, 1.0, 4.0, 8192)),
                                   dict(nh=2, nkv=2, d=10, dv=24, rot=0, base=10.0, sc=None),
                                   dict(nh=1, nkv=1, d=32, dv=32, rot=12, base=7.0, sc=None)])
 def test_projection_normed_over_all_heads_rotated_blended_and_stored(case):
@@ -153,9 +153,9 @@ def _paged(rng, k, v, B, dtype, keep_pages, passed):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [dict(nh=4, nkv=2, d=16, dv=24, B=16, W=20, K=3, cap=5.0), dict(nh=3, nkv=1, d=32, dv=32, B=8, W=33, K=21, cap=0.0),
-                                   dict(nh=2, nkv=2, d=10, dv=6, B=8, W=0, K=0, cap=2.0), dict(nh=2, nkv=1, d=64, dv=48, B=16, W=10, K=40, cap=30.0),
+                                   dict(nh=2, nkv=2, d=10, dv=6, B=8, W=0, K=0, cap=2.0), dict(nh=2, nkv=1, d=64, dv=40, B=16, W=10, K=40, cap=12.0),
                                    dict(nh=2, nkv=1, d=40, dv=40, B=32, W=1, K=2, cap=0.0), dict(nh=2, nkv=1, d=24, dv=24, B=16, W=70, K=70, cap=8.0),
-                                   dict(nh=2, nkv=2, d=64, dv=64, B=16, W=136, K=6, cap=30.0)])
+                                   dict(nh=2, nkv=2, d=64, dv=64, B=16, W=150, K=5, cap=25.0)])
 def test_window_attention_that_keeps_first_tokens_with_keys_that_stand_out_at_every_edge(shape, dtype):
     """One key is made to dominate the scores; it is put far away, at page borders, at the first position, on the last kept
     token and the one after it, just inside and just outside the window; decoded rows and runs of rows, through shuffled
