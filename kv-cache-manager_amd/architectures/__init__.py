@@ -3,3 +3,4 @@ from . import llama  # noqa: F401
 from . import kasuvik  # noqa: F401
 from . import furapel  # noqa: F401
 from . import fisesun  # noqa: F401
+from . import betirax  # noqa: F401

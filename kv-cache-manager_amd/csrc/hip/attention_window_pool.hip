@@ -6,7 +6,8 @@
 //                            blocks b with b*P + P - 1 <= i - window   (mean key, mean value of its P tokens)
 //                            tokens j < keep_first (the sequence's first tokens stay visible beyond the window)
 //   and all of them share one softmax; score = (q . k) * scale_h with a factor per query head, and with a cap c > 0
-//   score <- c tanh(score / c).
+//   score <- c tanh(score / c); then, with a slope per query head, score <- score - slope_h * (i - j) for token j (a bias
+//   that grows with the distance; not offered together with pooled blocks, which have no one distance).
 //
 // Pages: keys [pages, kv_heads, B, d], values transposed [pages, kv_heads, dv, B] (as the other
 // attentions of this library keep them).  Pooled entries are 32-bit and live with the page that holds
@@ -53,25 +54,30 @@ __global__ void rotary_freq_table_kernel(const int* __restrict__ positions, cons
 }
 
 // ------------------------------------------------------- rotation and the page write of a step
-// src [T, nh*d + nkv*d + nkv*dv] 32-bit (q | k | v).  q (rotated) -> q_out [T, nh*d]; k (rotated) and v
-// -> their page slot.  halves 0: the pair (2i, 2i+1), i < rot/2, is turned; halves 1: the pair (i, i + rot/2);
-// the rest passes.
+// src [T, nh*d + nkv*d + nkv*dv] 32-bit (q | k | v); or q alone there and (k | v) in rows of their own, kv_src
+// [T, nkv*d + nkv*dv] (a query that is made by a later product than the keys).  q (rotated) -> q_out [T, nh*d]; k
+// (rotated) and v -> their page slot; a row without a slot reads no k and no v.  halves 0: the pair (2i, 2i+1),
+// i < rot/2, is turned; halves 1: the pair (i, i + rot/2); the rest passes.
 template <class T>
 __global__ void __launch_bounds__(256)
-    rotate_store_kernel(const float* __restrict__ src, int ld, const float2* __restrict__ cos_sin, int rot, int halves,
+    rotate_store_kernel(const float* __restrict__ src, int ld, const float* __restrict__ kv_src, int ldkv,
+                        const float2* __restrict__ cos_sin, int rot, int halves,
                         const int* __restrict__ slots, T* __restrict__ q_out, int ldq, T* __restrict__ kcache,
                         T* __restrict__ vcache, int nh, int nkv, int d, int dv, int B) {
   const int row = blockIdx.x;
-  const float* r = src + size_t(row) * ld;
+  const float* rq = src + size_t(row) * ld;
+  const float* rk = kv_src ? kv_src + size_t(row) * ldkv : rq + size_t(nh) * d;      // (k | v) of the row
   const float2* cs = cos_sin + size_t(row) * (rot / 2);
   const int slot = slots ? slots[row] : -1;
-  for (int e = threadIdx.x; e < (nh + nkv) * d; e += blockDim.x) {
+  const int heads = slot >= 0 ? nh + nkv : nh;
+  for (int e = threadIdx.x; e < heads * d; e += blockDim.x) {
     const int head = e / d, i = e % d;
-    float x = r[e];
+    const float* r = head < nh ? rq + size_t(head) * d : rk + size_t(head - nh) * d;      // this head's entries
+    float x = r[i];
     if (i < rot) {      // rot is even: the partner lies inside the rotated part too
       const int hr = rot / 2;
       const bool second = halves ? i >= hr : (i & 1);
-      const float y = r[size_t(head) * d + (halves ? (second ? i - hr : i + hr) : (i ^ 1))];
+      const float y = r[halves ? (second ? i - hr : i + hr) : (i ^ 1)];
       const float2 a = cs[halves ? (second ? i - hr : i) : i / 2];
       x = second ? __fmaf_rn(x, a.x, __fmul_rn(y, a.y)) : __fmaf_rn(x, a.x, -__fmul_rn(y, a.y));
     }
@@ -79,7 +85,7 @@ __global__ void __launch_bounds__(256)
     else if (slot >= 0) store_f(kcache + ((size_t(slot / B) * nkv + (head - nh)) * B + slot % B) * d + i, x);
   }
   if (slot < 0) return;
-  const float* v = r + size_t(nh + nkv) * d;
+  const float* v = rk + size_t(nkv) * d;
   for (int e = threadIdx.x; e < nkv * dv; e += blockDim.x) {
     const int head = e / dv, i = e % dv;
     store_f(vcache + ((size_t(slot / B) * nkv + head) * dv + i) * B + slot % B, v[e]);
@@ -246,6 +252,7 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
                                  const float* __restrict__ pk, const float* __restrict__ pv,
                                  const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
                                  const int* __restrict__ ctx_lens, const float* __restrict__ head_scale,
+                                 const float* __restrict__ dist_slope,
                                  int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E, int keep_first,
                                  float softcap) {
   extern __shared__ float lds[];      // [d] q * scale * head_scale[h]; [waves][64] probabilities; [waves][dv + 2] results
@@ -277,6 +284,7 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
   const int head_chunks = block_chunks + (kept + kWave - 1) / kWave;
   const int first_chunk = first / kWave, chunks = head_chunks + ((ctx - 1) / kWave - first_chunk + 1);
   const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+  const float slope = dist_slope ? dist_slope[head] : 0.f;
   const bool wide_k = (d % N == 0) && (reinterpret_cast<uintptr_t>(kcache) % 16 == 0);
   const bool wide_pk = (d % 4 == 0);
   const bool wide_v = (B % N == 0) && (reinterpret_cast<uintptr_t>(vcache) % 16 == 0);
@@ -310,6 +318,7 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
       if (valid) s = dot_row<T>(qs, kcache + size_t(table[t / B]) * kpage + kvh * khead + size_t(t % B) * d, d, wide_k);
     }
     if (softcap > 0.f && valid) s = softcap * tanhf(s * inv_cap);
+    if (dist_slope && valid) s = fmaf(-slope, float(ctx - 1 - t), s);
     const float m_new = fmaxf(m, wave_max(s));
     const float alpha = expf(m - m_new);
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -432,21 +441,23 @@ int kvcm_rotary_freq_table(const int* positions, const double* freqs, float* cos
   return launch_status("rotary_freq_table");
 }
 
-int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, int halves, const int* slots, void* q_out, int dtype,
-                      int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B, hipStream_t s) {
+int kvcm_rotate_store(const float* src, int ld, const float* kv_src, int ldkv, const float* cos_sin, int rot, int halves,
+                      const int* slots, void* q_out, int dtype, int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d,
+                      int dv, int B, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && d > 0 && dv > 0 && B > 0, "rotate_store: bad sizes");
   KVCM_REQUIRE(rot % 2 == 0 && rot >= 0 && rot <= d, "rotate_store: %d rotated of %d dims is not supported "
                "(an even number, at most the head's size)", rot, d);
   KVCM_REQUIRE(rot == 0 || cos_sin != nullptr, "rotate_store: a rotation needs its table");
-  KVCM_REQUIRE(ld >= (nh + nkv) * d + nkv * dv && ldq >= nh * d, "rotate_store: row strides too small");
+  if (kv_src) KVCM_REQUIRE(ld >= nh * d && ldkv >= nkv * (d + dv) && ldq >= nh * d, "rotate_store: row strides too small");
+  else KVCM_REQUIRE(ld >= (slots ? (nh + nkv) * d + nkv * dv : nh * d) && ldq >= nh * d, "rotate_store: row strides too small");
   KVCM_REQUIRE(!slots || (kcache && vcache), "rotate_store: slots without pages");
   const float2* cs = reinterpret_cast<const float2*>(cos_sin);
   if (dtype == kF32)
-    rotate_store_kernel<float><<<T, 256, 0, s>>>(src, ld, cs, rot, halves, slots, static_cast<float*>(q_out), ldq,
+    rotate_store_kernel<float><<<T, 256, 0, s>>>(src, ld, kv_src, ldkv, cs, rot, halves, slots, static_cast<float*>(q_out), ldq,
                                                   static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, d, dv, B);
   else if (dtype == kBF16)
-    rotate_store_kernel<bf16_t><<<T, 256, 0, s>>>(src, ld, cs, rot, halves, slots, static_cast<bf16_t*>(q_out), ldq,
+    rotate_store_kernel<bf16_t><<<T, 256, 0, s>>>(src, ld, kv_src, ldkv, cs, rot, halves, slots, static_cast<bf16_t*>(q_out), ldq,
                                                    static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, d, dv, B);
   else KVCM_REQUIRE(false, "rotate_store: unknown dtype %d", dtype);
   return launch_status("rotate_store");
@@ -499,8 +510,9 @@ int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* p
 
 int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
-                               const int* ctx_lens, const float* head_scale, int T, int nh, int nkv, int d, int dv, int B,
-                               float scale, int window, int P, int E, int keep_first, float softcap, hipStream_t s) {
+                               const int* ctx_lens, const float* head_scale, const float* dist_slope, int T, int nh, int nkv,
+                               int d, int dv, int B, float scale, int window, int P, int E, int keep_first, float softcap,
+                               hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && B > 0 && d > 0, "attention_window_pool: bad sizes T=%d heads=%d kv_heads=%d", T, nh, nkv);
   KVCM_REQUIRE(nh % nkv == 0, "attention_window_pool: %d query heads are not a multiple of %d kv heads", nh, nkv);
@@ -510,19 +522,20 @@ int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int
   KVCM_REQUIRE(window >= 0 && P >= 0, "attention_window_pool: negative window or block");
   KVCM_REQUIRE(P == 0 || (pk && pv && E == (B + P - 1) / P), "attention_window_pool: pooled blocks need their entries");
   KVCM_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attention_window_pool: negative count of kept tokens or score cap");
+  KVCM_REQUIRE(!dist_slope || P == 0, "attention_window_pool: a distance bias beside pooled blocks is not supported");
   const long long blocks = static_cast<long long>(T) * nh;
   KVCM_REQUIRE(blocks < (1ll << 31), "attention_window_pool: too many rows");
   const size_t lds = sizeof(float) * (d + kWpWaves * kWave + kWpWaves * (dv + 2));
   if (dtype == kF32)
     attention_window_pool_kernel<float><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
         static_cast<const float*>(q), ldq, static_cast<float*>(out), ldo, static_cast<const float*>(kcache),
-        static_cast<const float*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, nh, nkv, d, dv,
-        B, scale, window, P, E, keep_first, softcap);
+        static_cast<const float*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, dist_slope, nh,
+        nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   else if (dtype == kBF16)
     attention_window_pool_kernel<bf16_t><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
         static_cast<const bf16_t*>(q), ldq, static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(kcache),
-        static_cast<const bf16_t*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, nh, nkv, d, dv,
-        B, scale, window, P, E, keep_first, softcap);
+        static_cast<const bf16_t*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, dist_slope, nh,
+        nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   else KVCM_REQUIRE(false, "attention_window_pool: unknown dtype %d", dtype);
   return launch_status("attention_window_pool");
 }

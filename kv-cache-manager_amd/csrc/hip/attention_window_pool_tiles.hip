@@ -8,7 +8,8 @@
 // (window, causality, blocks wholly before the window), so a chunk that some rows of the tile do not see
 // costs them nothing but zeros; a row's chunks and their order depend on its own position only.  The first
 // keep_first tokens of a sequence may stay visible beyond the window (chunks of their own, from token 0), and the
-// scores may be capped, score <- c tanh(score / c).
+// scores may be capped, score <- c tanh(score / c), and a bias that grows with the distance may be taken off them,
+// score <- score - slope_h * (i - j) with a slope per query head (tokens only: not beside pooled blocks).
 // bfloat16 storage only; sizes d and dv in multiples of 8, pages whose size is a multiple of 8 and divides 64.
 #include <cfloat>
 
@@ -34,7 +35,8 @@ __global__ void __launch_bounds__(256)
                                        const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                                        const float* __restrict__ pk, const float* __restrict__ pv,
                                        const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
-                                       const int* __restrict__ seq_start, const float* __restrict__ head_scale, int tiles_per_seq,
+                                       const int* __restrict__ seq_start, const float* __restrict__ head_scale,
+                                       const float* __restrict__ dist_slope, int tiles_per_seq,
                                        int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E,
                                        int keep_first, float softcap) {
   constexpr int KP = DP + 8, KS = DP / 32, DVP = DVT * 16;
@@ -58,6 +60,7 @@ __global__ void __launch_bounds__(256)
   constexpr float kLog2e = 1.44269504088896341f;
   const float f = (head_scale ? scale * head_scale[head] : scale) * (softcap > 0.f ? 1.0f / softcap : kLog2e);
   const float cap2 = softcap * kLog2e;
+  const float slope2 = dist_slope ? dist_slope[head] * kLog2e : 0.f;      // the bias in units of log 2, like the scores
 
   // this wave's 16 query rows as first operands (row = lane % 16, k = 8 * (lane / 16) .. + 8 of every 32)
   bf16x8 qf[KS];
@@ -201,6 +204,7 @@ __global__ void __launch_bounds__(256)
                           : (key >= t_lo && key <= pos[i] && (window == 0 || key > pos[i] - window || key < keep_first));
         float sv = sc[ct][i] * f;
         if (softcap > 0.f) sv = cap2 * tanhf(sv);
+        if (dist_slope) sv = fmaf(-slope2, float(pos[i] - key), sv);
         sv = vis[ct] ? sv : kMasked;
         sc[ct][i] = sv;
         mx = fmaxf(mx, sv);
@@ -252,12 +256,12 @@ __global__ void __launch_bounds__(256)
 template <int DP>
 int launch_tiles(int dvt, dim3 grid, hipStream_t s, const uint16_t* q, int ldq, uint16_t* out, int ldo, const uint16_t* kc,
                  const uint16_t* vc, const float* pk, const float* pv, const int* tables, int table_stride, const int* run_start,
-                 const int* seq_start, const float* head_scale, int tiles_per_seq, int nh, int nkv, int d, int dv, int B,
-                 float scale, int window, int P, int E, int keep_first, float softcap) {
+                 const int* seq_start, const float* head_scale, const float* dist_slope, int tiles_per_seq, int nh, int nkv, int d,
+                 int dv, int B, float scale, int window, int P, int E, int keep_first, float softcap) {
 #define KVCM_TILES(DVT)                                                                                                     \
   attention_window_pool_tiles_kernel<DP, DVT><<<grid, 256, 0, s>>>(q, ldq, out, ldo, kc, vc, pk, pv, tables, table_stride,   \
-                                                                   run_start, seq_start, head_scale, tiles_per_seq, nh, nkv, \
-                                                                   d, dv, B, scale, window, P, E, keep_first, softcap)
+                                                                   run_start, seq_start, head_scale, dist_slope, tiles_per_seq, \
+                                                                   nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap)
   if (dvt <= 2) KVCM_TILES(2);
   else if (dvt <= 4) KVCM_TILES(4);
   else if (dvt <= 8) KVCM_TILES(8);
@@ -279,9 +283,9 @@ int kvcm_attention_window_pool_tiles_supported(int d, int dv, int B) {
 // q, out, pages: bfloat16; pooled entries: 32-bit.  S sequences with runs of up to max_run rows.
 int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                      const float* pk, const float* pv, const int* tables, int table_stride,
-                                     const int* run_start, const int* seq_start, const float* head_scale, int S, int max_run,
-                                     int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E,
-                                     int keep_first, float softcap, hipStream_t s) {
+                                     const int* run_start, const int* seq_start, const float* head_scale, const float* dist_slope,
+                                     int S, int max_run, int nh, int nkv, int d, int dv, int B, float scale, int window, int P,
+                                     int E, int keep_first, float softcap, hipStream_t s) {
   if (S == 0 || max_run == 0) return 0;
   KVCM_REQUIRE(S > 0 && max_run > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_window_pool_tiles: bad sizes");
   KVCM_REQUIRE(kvcm_attention_window_pool_tiles_supported(d, dv, B),
@@ -292,6 +296,7 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
                "attention_window_pool_tiles: pooled blocks need their entries");
   KVCM_REQUIRE(P == 0 || d % 8 == 0, "attention_window_pool_tiles: pooled keys are read eight at a time");
   KVCM_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attention_window_pool_tiles: negative count of kept tokens or score cap");
+  KVCM_REQUIRE(!dist_slope || P == 0, "attention_window_pool_tiles: a distance bias beside pooled blocks is not supported");
   const int tiles_per_seq = (max_run + kTileRows - 1) / kTileRows;
   KVCM_REQUIRE(static_cast<long long>(S) * tiles_per_seq < (1ll << 31) && nh <= 65535, "attention_window_pool_tiles: too many rows");
   const dim3 grid(S * tiles_per_seq, nh);
@@ -302,12 +307,12 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
   const uint16_t* vc = static_cast<const uint16_t*>(vcache);
   if (d <= 32)
     return launch_tiles<32>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                            tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
+                            dist_slope, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   if (d <= 64)
     return launch_tiles<64>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                            tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
+                            dist_slope, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   return launch_tiles<128>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                           tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
+                           dist_slope, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
 }
 
 }  // extern "C"

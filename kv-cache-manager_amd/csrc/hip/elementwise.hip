@@ -458,6 +458,21 @@ __global__ void __launch_bounds__(256)
   store_f(out + size_t(t) * ldo + i, a * u);
 }
 
+// out[t, i] = act(in[t, i]) for feed-forwards without a gate: the same activations, computed in 32-bit, rounded once.
+template <class TO>
+__global__ void __launch_bounds__(256)
+    act_rows_kernel(const float* __restrict__ in, int ld, TO* __restrict__ out, int ldo, int I, int act) {
+  const int t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= I) return;
+  const float g = in[size_t(t) * ld + i];
+  float a;
+  if (act == 1) a = fmaxf(g, 0.f);
+  else if (act == 2) a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  else a = g / (1.0f + expf(-g));
+  store_f(out + size_t(t) * ldo + i, a);
+}
+
 
 }  // namespace kvcm
 
@@ -487,6 +502,18 @@ int kvcm_gated_act(const float* gate_up, int ld, void* out, int out_dtype, int l
   else if (out_dtype == kBF16) gated_act_kernel<bf16_t><<<grid, 256, 0, s>>>(gate_up, ld, static_cast<bf16_t*>(out), ldo, I, act);
   else KVCM_REQUIRE(false, "gated_act: unknown output dtype %d", out_dtype);
   return launch_status("gated_act");
+}
+
+int kvcm_act_rows(const float* in, int ld, void* out, int out_dtype, int ldo, int T, int I, int act, hipStream_t s) {
+  if (T == 0) return 0;
+  KVCM_REQUIRE(T > 0 && I > 0 && ld >= I && ldo >= I && in && out, "act_rows: bad sizes T=%d I=%d", T, I);
+  KVCM_REQUIRE(T <= 65535, "act_rows: too many rows for one launch (%d)", T);
+  KVCM_REQUIRE(act >= 0 && act <= 2, "act_rows: unknown activation %d (0 silu, 1 relu, 2 gelu_tanh)", act);
+  const dim3 grid((I + 255) / 256, T);
+  if (out_dtype == kF32) act_rows_kernel<float><<<grid, 256, 0, s>>>(in, ld, static_cast<float*>(out), ldo, I, act);
+  else if (out_dtype == kBF16) act_rows_kernel<bf16_t><<<grid, 256, 0, s>>>(in, ld, static_cast<bf16_t*>(out), ldo, I, act);
+  else KVCM_REQUIRE(false, "act_rows: unknown output dtype %d", out_dtype);
+  return launch_status("act_rows");
 }
 
 int kvcm_embed(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V, hipStream_t s) {

@@ -169,15 +169,17 @@ int kvcm_short_conv_state(const float* in, int ld_in, const float* bias_in, floa
 int kvcm_rotary_pairs_table(const int* positions, float* cos_sin, int T, int dims, float base, hipStream_t s);
 int kvcm_rotary_freq_table(const int* positions, const double* freqs, float* cos_sin, int T, int dims, float factor,
                            hipStream_t s);
-int kvcm_rotate_store(const float* src, int ld, const float* cos_sin, int rot, int halves, const int* slots, void* q_out, int dtype,
-                      int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B, hipStream_t s);
+int kvcm_rotate_store(const float* src, int ld, const float* kv_src, int ldkv, const float* cos_sin, int rot, int halves,
+                      const int* slots, void* q_out, int dtype, int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d,
+                      int dv, int B, hipStream_t s);
 int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* pk, float* pv, const int* tables,
                      int table_stride, const int* row_seq, const int* positions, const int* slots, int T, int nkv, int d,
                      int dv, int B, int P, int E, hipStream_t s);
 int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
-                               const int* ctx_lens, const float* head_scale, int T, int nh, int nkv, int d, int dv, int B,
-                               float scale, int window, int P, int E, int keep_first, float softcap, hipStream_t s);
+                               const int* ctx_lens, const float* head_scale, const float* dist_slope, int T, int nh, int nkv,
+                               int d, int dv, int B, float scale, int window, int P, int E, int keep_first, float softcap,
+                               hipStream_t s);
 // as rotate_store, after q and k were divided by the root mean square of their whole stretch (times a weight) and v was
 // blended with another layer's values of the same row
 int kvcm_norm_rotate_store(const float* src, int ld, const float* wq, const float* wk, float eps, const float* v_other, int ldvo,
@@ -188,9 +190,9 @@ int kvcm_norm_rotate_store(const float* src, int ld, const float* wq, const floa
 int kvcm_attention_window_pool_tiles_supported(int d, int dv, int B);
 int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                      const float* pk, const float* pv, const int* tables, int table_stride,
-                                     const int* run_start, const int* seq_start, const float* head_scale, int S, int max_run,
-                                     int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E,
-                                     int keep_first, float softcap, hipStream_t s);
+                                     const int* run_start, const int* seq_start, const float* head_scale, const float* dist_slope,
+                                     int S, int max_run, int nh, int nkv, int d, int dv, int B, float scale, int window, int P,
+                                     int E, int keep_first, float softcap, hipStream_t s);
 // (selective_scan.hip, delta_rule.hip) recurrences with a 32-bit state per sequence
 int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, int lddt, const float* dt_bias,
                         const float* bc, int ldbc, int off_b, int off_c, const float* a_log, const float* dskip,
@@ -215,8 +217,20 @@ int kvcm_stream_pack(const float* x, const float* a, const float* b, const float
                      hipStream_t s);
 int kvcm_scale_rows(float* x, long long n, float factor, hipStream_t s);
 int kvcm_softcap_rows(float* x, long long n, float cap, hipStream_t s);
-int kvcm_head_gate(void* o, int dtype, int ldo, const float* gate, int ldg, int T, int heads, int dv, hipStream_t s);
-int kvcm_rms_groups(float* x, int ld, int col0, int size, int groups, const float* w, float eps, int T, hipStream_t s);
+int kvcm_head_gate(void* o, int dtype, int ldo, const float* gate, int ldg, int T, int heads, int dv, int per_element, hipStream_t s);
+int kvcm_rms_groups(float* x, int ld, int col0, int size, int groups, const float* w, float eps, void* out, int out_dtype, int ldo,
+                    int T, hipStream_t s);
+// (post_norm.hip) layers that norm after the sum; an attention's norm per head with biases, a query temperature and the page write
+int kvcm_layernorm_post(float* x, const float* a, int a_splits, long long split_stride, const float* bias, float alpha,
+                        const float* weight, const int* rows, void* out, int out_dtype, int R, int H, float eps, hipStream_t s);
+int kvcm_head_norm_store(const float* src, int ld, const float* bias, const float* wq, const float* wk, float eps,
+                         const int* positions, float temp_coef, int temp_every, int values_are_keys, const int* slots, void* q_out,
+                         int dtype, int ldq, void* kcache, void* vcache, int T, int nh, int nkv, int d, int dv, int B, hipStream_t s);
+// (gemm_heads.hip) one small product per head in one launch, with an optional sigmoid gate per element
+int kvcm_gemm_heads(const void* X, int in_dtype, int ldx, const void* W, void* Y, int out_dtype, int ldy, const float* gate,
+                    int ldg, int M, int heads, int N, int K, hipStream_t s);
+// (elementwise.hip) an activation without a gate on 32-bit rows
+int kvcm_act_rows(const float* in, int ld, void* out, int out_dtype, int ldo, int T, int I, int act, hipStream_t s);
 // (mlstm.hip) a matrix memory with exponential gates, walked token by token
 int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* ig, int ldi,
                     const float* fg, int ldf, const float* i_bias, const float* f_bias, float cap, float q_scale, float* coef,
@@ -224,7 +238,7 @@ int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const floa
                     const int* seq_start, const int* state_slots, int S, int heads, int dk, int dv, int T, int max_run,
                     hipStream_t s);
 // (moe.hip) a routed feed-forward: the choice of experts, and the experts' two products a row at a time
-int kvcm_moe_route(const float* logits, int ld, int E, int top, int* chosen, float* weight, int T, hipStream_t s);
+int kvcm_moe_route(const float* logits, int ld, int E, int top, int over_chosen, int* chosen, float* weight, int T, hipStream_t s);
 int kvcm_moe_table_route(const int* tokens, const int* table, int vocab, int ld, int top, int* chosen, float* weight, int T,
                          hipStream_t s);
 int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* chosen, void* act, int T, int K, int F, int top,

@@ -2,7 +2,8 @@
 // sum of their outputs weighted by the chosen scores as they are (not renormalized).
 //
 //   moe_route      32-bit router logits [T, E] -> chosen[T, top] (expert numbers, best first; equal scores: the lower
-//                  number) and weight[T, top] (their softmax scores over all E).  One wave per row.
+//                  number) and weight[T, top]: their softmax scores over all E, or (over_chosen) the softmax over the
+//                  chosen logits alone, which add up to one.  One wave per row.
 //   moe_table_route  chosen[T, top] = table[token of the row, :] (a table of expert numbers per token id), weight = 1 / top
 //   moe_up         act[T, top, F] = a(W_up[e] h) for each row's chosen experts, a = square of relu, rounded to the
 //                  compute dtype; or, gated, act = silu(W_gate[e] h) * (W_up[e] h) with the two matrices of an expert
@@ -24,7 +25,7 @@ namespace kvcm {
 constexpr int kMoeMaxTop = 16;
 
 __global__ void __launch_bounds__(256)
-    moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top, int* __restrict__ chosen,
+    moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top, int over_chosen, int* __restrict__ chosen,
                      float* __restrict__ weight, int T) {
   const int row = blockIdx.x * (256 / kWave) + threadIdx.x / kWave, lane = threadIdx.x % kWave;
   if (row >= T) return;
@@ -37,6 +38,7 @@ __global__ void __launch_bounds__(256)
   sum = wave_sum(sum);
   const float inv = 1.0f / sum;
   int taken[kMoeMaxTop];
+  float picked[kMoeMaxTop];
   for (int s = 0; s < top; ++s) {
     float best = -FLT_MAX;
     int at = 0x7fffffff;
@@ -53,10 +55,17 @@ __global__ void __launch_bounds__(256)
       if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
     }
     taken[s] = at;
+    picked[s] = expf(best - mx);      // the first pick is the largest logit: exp(0)
     if (lane == 0) {
       chosen[size_t(row) * top + s] = at;
-      weight[size_t(row) * top + s] = expf(best - mx) * inv;
+      if (!over_chosen) weight[size_t(row) * top + s] = picked[s] * inv;
     }
+  }
+  if (over_chosen && lane == 0) {
+    float among = 0.f;
+    for (int s = 0; s < top; ++s) among += picked[s];
+    const float inv_among = 1.0f / among;
+    for (int s = 0; s < top; ++s) weight[size_t(row) * top + s] = picked[s] * inv_among;
   }
 }
 
@@ -211,11 +220,11 @@ using namespace kvcm;
 
 extern "C" {
 
-int kvcm_moe_route(const float* logits, int ld, int E, int top, int* chosen, float* weight, int T, hipStream_t s) {
+int kvcm_moe_route(const float* logits, int ld, int E, int top, int over_chosen, int* chosen, float* weight, int T, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E && ld >= E, "moe_route: bad sizes T=%d experts=%d top=%d", T, E, top);
   KVCM_REQUIRE(top <= kMoeMaxTop, "moe_route: %d experts a row are not supported (up to %d)", top, kMoeMaxTop);
-  moe_route_kernel<<<(T + 3) / 4, 256, 0, s>>>(logits, ld, E, top, chosen, weight, T);
+  moe_route_kernel<<<(T + 3) / 4, 256, 0, s>>>(logits, ld, E, top, over_chosen, chosen, weight, T);
   return launch_status("moe_route");
 }
 

@@ -120,6 +120,10 @@ const Entry kEntries[] = {
     KVCM_ENTRY(kvcm_scan_prepare),
     KVCM_ENTRY(kvcm_delta_prepare),
     KVCM_ENTRY(kvcm_delta_scan),
+    KVCM_ENTRY(kvcm_layernorm_post),
+    KVCM_ENTRY(kvcm_head_norm_store),
+    KVCM_ENTRY(kvcm_gemm_heads),
+    KVCM_ENTRY(kvcm_act_rows),
 };
 #undef KVCM_ENTRY
 

@@ -7,9 +7,10 @@
 //   stream_pack    [x + a + b | x0] as rows of the compute dtype: the input of a product that mixes the stream
 //                  with the embedding again
 //   scale_rows     32-bit values times a factor, in place (a head's logit scale)
-//   head_gate      an attention's output times one sigmoid gate per (row, head), in place
+//   head_gate      an attention's output times one sigmoid gate per (row, head), or one per element, in place
 //   rms_groups     32-bit rows: groups of consecutive columns divided by their root mean square and weighted,
-//                  in place (the small latent vector that a latent attention keeps per token)
+//                  in place (the small latent vector that a latent attention keeps per token) or into rows of the
+//                  compute dtype (a latent that the next product reads)
 //
 // Everything here is 32-bit arithmetic on 32-bit inputs; only the outputs that feed products are rounded.
 #include "common.h"
@@ -65,21 +66,23 @@ __global__ void __launch_bounds__(256) softcap_rows_kernel(float* __restrict__ x
 
 template <class T>
 __global__ void __launch_bounds__(256)
-    head_gate_kernel(T* __restrict__ o, int ldo, const float* __restrict__ gate, int ldg, long long n, int heads, int dv) {
+    head_gate_kernel(T* __restrict__ o, int ldo, const float* __restrict__ gate, int ldg, long long n, int heads, int dv,
+                     int per_element) {
   const int per_row = heads * dv;
   for (long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x; idx < n; idx += static_cast<long long>(gridDim.x) * 256) {
     const long long r = idx / per_row;
     const int c = static_cast<int>(idx % per_row);
-    const float g = 1.0f / (1.0f + expf(-gate[r * ldg + c / dv]));
+    const float g = 1.0f / (1.0f + expf(-gate[r * ldg + (per_element ? c : c / dv)]));
     T* p = o + r * ldo + c;
     store_f(p, load_f(p) * g);
   }
 }
 
-// one wave per (row, group)
+// one wave per (row, group); out null: in place, else out[row, g * size + i] in TO
+template <class TO>
 __global__ void __launch_bounds__(256)
     rms_groups_kernel(float* __restrict__ x, int ld, int col0, int size, int groups, const float* __restrict__ w, float eps,
-                      long long items) {
+                      TO* __restrict__ out, int ldo, long long items) {
   const long long item = static_cast<long long>(blockIdx.x) * (256 / kWave) + threadIdx.x / kWave;
   if (item >= items) return;
   const int lane = threadIdx.x % kWave;
@@ -88,7 +91,12 @@ __global__ void __launch_bounds__(256)
   for (int i = lane; i < size; i += kWave) ss = fmaf(p[i], p[i], ss);
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / float(size) + eps);
-  for (int i = lane; i < size; i += kWave) p[i] = p[i] * inv * w[i];
+  if (out) {
+    TO* q = out + (item / groups) * ldo + (item % groups) * size;
+    for (int i = lane; i < size; i += kWave) store_f(q + i, p[i] * inv * w[i]);
+  } else {
+    for (int i = lane; i < size; i += kWave) p[i] = p[i] * inv * w[i];
+  }
 }
 
 inline unsigned grid_for(long long n) {
@@ -153,27 +161,34 @@ int kvcm_softcap_rows(float* x, long long n, float cap, hipStream_t s) {
   return launch_status("softcap_rows");
 }
 
-// o [T, heads*dv] (dtype) *= sigmoid(gate[T, heads]) per head
-int kvcm_head_gate(void* o, int dtype, int ldo, const float* gate, int ldg, int T, int heads, int dv, hipStream_t s) {
+// o [T, heads*dv] (dtype) *= sigmoid(gate[T, heads]) per head, or (per_element) sigmoid(gate[T, heads*dv]) per element
+int kvcm_head_gate(void* o, int dtype, int ldo, const float* gate, int ldg, int T, int heads, int dv, int per_element, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && heads > 0 && dv > 0 && o && gate, "head_gate: bad sizes");
-  KVCM_REQUIRE(ldo >= heads * dv && ldg >= heads, "head_gate: row strides too small");
+  KVCM_REQUIRE(ldo >= heads * dv && ldg >= (per_element ? heads * dv : heads), "head_gate: row strides too small");
   const long long n = static_cast<long long>(T) * heads * dv;
-  if (dtype == kF32) head_gate_kernel<float><<<grid_for(n), 256, 0, s>>>(static_cast<float*>(o), ldo, gate, ldg, n, heads, dv);
-  else if (dtype == kBF16) head_gate_kernel<bf16_t><<<grid_for(n), 256, 0, s>>>(static_cast<bf16_t*>(o), ldo, gate, ldg, n, heads, dv);
+  if (dtype == kF32) head_gate_kernel<float><<<grid_for(n), 256, 0, s>>>(static_cast<float*>(o), ldo, gate, ldg, n, heads, dv, per_element);
+  else if (dtype == kBF16) head_gate_kernel<bf16_t><<<grid_for(n), 256, 0, s>>>(static_cast<bf16_t*>(o), ldo, gate, ldg, n, heads, dv, per_element);
   else KVCM_REQUIRE(false, "head_gate: unknown dtype %d", dtype);
   return launch_status("head_gate");
 }
 
-// x [T, ld]: columns col0 + g*size .. + size, g < groups, each <- n(.) * w[0..size)
-int kvcm_rms_groups(float* x, int ld, int col0, int size, int groups, const float* w, float eps, int T, hipStream_t s) {
+// x [T, ld]: columns col0 + g*size .. + size, g < groups, each <- n(.) * w[0..size); with out: x stays and
+// out [T, ldo] (out_dtype) receives the groups side by side from its column 0
+int kvcm_rms_groups(float* x, int ld, int col0, int size, int groups, const float* w, float eps, void* out, int out_dtype, int ldo,
+                    int T, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && size > 0 && groups > 0 && col0 >= 0 && x && w, "rms_groups: bad sizes");
   KVCM_REQUIRE(ld >= col0 + size * groups, "rms_groups: the groups do not fit the rows");
+  KVCM_REQUIRE(!out || ldo >= size * groups, "rms_groups: the groups do not fit the output's rows");
   const long long items = static_cast<long long>(T) * groups;
   const long long blocks = (items + 3) / 4;
   KVCM_REQUIRE(blocks < (1ll << 31), "rms_groups: too many rows");
-  rms_groups_kernel<<<static_cast<unsigned>(blocks), 256, 0, s>>>(x, ld, col0, size, groups, w, eps, items);
+  if (!out || out_dtype == kF32)
+    rms_groups_kernel<float><<<static_cast<unsigned>(blocks), 256, 0, s>>>(x, ld, col0, size, groups, w, eps, static_cast<float*>(out), ldo, items);
+  else if (out_dtype == kBF16)
+    rms_groups_kernel<bf16_t><<<static_cast<unsigned>(blocks), 256, 0, s>>>(x, ld, col0, size, groups, w, eps, static_cast<bf16_t*>(out), ldo, items);
+  else KVCM_REQUIRE(false, "rms_groups: unknown output dtype %d", out_dtype);
   return launch_status("rms_groups");
 }
 

@@ -96,17 +96,21 @@ def _declare(lib):
     fn("kvcm_short_conv", vp, i, vp, vp, vp, vp, vp, i, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
     fn("kvcm_short_conv_state", vp, i, vp, vp, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_rotary_pairs_table", vp, vp, i, i, f, vp)
-    fn("kvcm_rotate_store", vp, i, vp, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_rotate_store", vp, i, vp, i, vp, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_norm_rotate_store", vp, i, vp, vp, f, vp, i, f, vp, i, vp, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_rotary_freq_table", vp, vp, vp, i, i, f, vp)
     fn("kvcm_dyt_norm", vp, i, vp, i, C.c_longlong, vp, vp, i, vp, vp, f, vp, vp, vp, f, vp, i, i, i, vp)
     fn("kvcm_stream_pack", vp, vp, vp, vp, vp, i, i, i, vp)
     fn("kvcm_scale_rows", vp, C.c_longlong, f, vp)
     fn("kvcm_softcap_rows", vp, C.c_longlong, f, vp)
-    fn("kvcm_head_gate", vp, i, i, vp, i, i, i, i, vp)
-    fn("kvcm_rms_groups", vp, i, i, i, i, vp, f, i, vp)
+    fn("kvcm_head_gate", vp, i, i, vp, i, i, i, i, i, vp)
+    fn("kvcm_rms_groups", vp, i, i, i, i, vp, f, vp, i, i, i, vp)
+    fn("kvcm_layernorm_post", vp, vp, i, C.c_longlong, vp, f, vp, vp, vp, i, i, i, f, vp)
+    fn("kvcm_head_norm_store", vp, i, vp, vp, vp, f, vp, f, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
+    fn("kvcm_gemm_heads", vp, i, i, vp, vp, i, i, vp, i, i, i, i, i, vp)
+    fn("kvcm_act_rows", vp, i, vp, i, i, i, i, i, vp)
     fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
-    fn("kvcm_moe_route", vp, i, i, i, vp, vp, i, vp)
+    fn("kvcm_moe_route", vp, i, i, i, i, vp, vp, i, vp)
     fn("kvcm_moe_table_route", vp, vp, i, i, i, vp, vp, i, vp)
     fn("kvcm_moe_up", vp, i, i, vp, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_moe_down", vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
@@ -114,9 +118,9 @@ def _declare(lib):
     fn("kvcm_moe_grouped_max_tiles", i, i)
     fn("kvcm_moe_grouped", vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_pool_update", vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp)
-    fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, f, vp)
+    fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, f, vp)
     fn("kvcm_attention_window_pool_tiles_supported", i, i, i)
-    fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, i, f, vp)
+    fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, i, f, vp)
     fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, i, vp)
     fn("kvcm_scan_prepare", vp, i, vp, vp, i, i, i, vp)
     fn("kvcm_delta_prepare", vp, i, vp, i, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
@@ -1109,12 +1113,19 @@ def rotary_pairs_table(positions, out, dims, base, rows=None):
     return out
 
 
-def rotate_store(qkv, q_out, nh, nkv, d, dv, cos_sin=None, rot=0, slots=None, kcache=None, vcache=None, rows=None, halves=False):
-    """qkv: 32-bit rows [q (nh*d) | k (nkv*d) | v (nkv*dv)].  The first ``rot`` entries of every q and k head are
+def rotate_store(qkv, q_out, nh, nkv, d, dv, cos_sin=None, rot=0, slots=None, kcache=None, vcache=None, rows=None, halves=False,
+                 kv=None):
+    """qkv: 32-bit rows [q (nh*d) | k (nkv*d) | v (nkv*dv)]; or q alone there and ``kv``: 32-bit rows [k | v] of their
+    own; without ``slots`` only q is read.  The first ``rot`` entries of every q and k head are
     turned with the table ``cos_sin``, by interleaved pairs (2i, 2i+1) or, with ``halves``, by pairs (i, i + rot/2);
     q goes to q_out [T, nh*d], k and v to their page slots (keys [pages, nkv, B, d], values [pages, nkv, dv, B])."""
     T = q_out.shape[0] if rows is None else rows
-    _f32rows(qkv, "qkv", (nh + nkv) * d + nkv * dv)
+    if kv is not None:
+        _f32rows(qkv, "q", nh * d)
+        _f32rows(kv, "kv", nkv * (d + dv))
+        _need(kv.shape[0] >= T, "rotate_store: kv has fewer rows than the step")
+    else:
+        _f32rows(qkv, "qkv", (nh + nkv) * d + nkv * dv if slots is not None else nh * d)
     _rows2d(q_out, "q_out")
     _need(q_out.shape[1] >= nh * d and q_out.is_cuda and qkv.shape[0] >= T, "rotate_store: shapes do not agree")
     B = 1
@@ -1128,7 +1139,7 @@ def rotate_store(qkv, q_out, nh, nkv, d, dv, cos_sin=None, rot=0, slots=None, kc
     if rot:
         _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.numel() >= T * rot,
               "cos_sin must be float32 [rows, rot/2, 2]")
-    _call("kvcm_rotate_store", _ptr(qkv), qkv.stride(0), _ptr(cos_sin), rot, 1 if halves else 0, _ptr(slots), _ptr(q_out), _DT[q_out.dtype],
+    _call("kvcm_rotate_store", _ptr(qkv), qkv.stride(0), _ptr(kv), kv.stride(0) if kv is not None else 0, _ptr(cos_sin), rot, 1 if halves else 0, _ptr(slots), _ptr(q_out), _DT[q_out.dtype],
           q_out.stride(0), _ptr(kcache), _ptr(vcache), T, nh, nkv, d, dv, B, _stream())
 
 
@@ -1196,10 +1207,11 @@ def pool_update(kcache, vcache, pk, pv, tables, table_stride, row_seq, positions
 
 
 def attention_window_pool(q, out, kcache, vcache, pk, pv, tables, table_stride, row_seq, ctx_lens, nh, nkv, d, dv, scale,
-                          window, P, head_scale=None, rows=None, keep_first=0, softcap=0.0):
+                          window, P, head_scale=None, rows=None, keep_first=0, softcap=0.0, dist_slope=None):
     """out[r, h] = softmax over the last ``window`` tokens, the sequence's first ``keep_first`` tokens and the pooled
     blocks of P tokens before the window (window 0: every token, no blocks) of (q . k) * scale * head_scale[h], times the
-    values.  ``softcap`` c > 0: the scores are capped first, c tanh(score / c)."""
+    values.  ``softcap`` c > 0: the scores are capped first, c tanh(score / c).  ``dist_slope`` (float32 [nh]): a bias that
+    grows with the distance is taken off the scores, slope[h] * (query position - key position)."""
     _dev(q, out, kcache, vcache, tables, row_seq, ctx_lens)
     _rows2d(q, "q")
     _rows2d(out, "out")
@@ -1208,11 +1220,12 @@ def attention_window_pool(q, out, kcache, vcache, pk, pv, tables, table_stride, 
     _need(q.shape[1] >= nh * d and out.shape[1] >= nh * dv, "attention rows are too short for the head layout")
     B, E = _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P)
     _f32(head_scale, "head_scale", nh)
+    _f32(dist_slope, "dist_slope", nh)
     _i32(row_seq, "row_seq", T)
     _i32(ctx_lens, "ctx_lens", T)
     _i32(tables, "tables")
     _call("kvcm_attention_window_pool", _ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
-          _ptr(pk), _ptr(pv), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), _ptr(head_scale), T, nh, nkv, d, dv,
+          _ptr(pk), _ptr(pv), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), _ptr(head_scale), _ptr(dist_slope), T, nh, nkv, d, dv,
           B, float(scale), int(window), int(P), E, int(keep_first), float(softcap or 0.0), _stream())
 
 
@@ -1222,7 +1235,7 @@ def attention_window_pool_tiles_supported(d, dv, dtype, block_size):
 
 
 def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_stride, run_start, seq_start, num_seqs, max_run,
-                                nh, nkv, d, dv, scale, window, P, head_scale=None, keep_first=0, softcap=0.0):
+                                nh, nkv, d, dv, scale, window, P, head_scale=None, keep_first=0, softcap=0.0, dist_slope=None):
     """``attention_window_pool`` for steps whose sequences run several consecutive positions: 64 rows of a run and one
     head per workgroup on the matrix cores (bfloat16 only).  Every row of every run is computed, single rows too."""
     _dev(q, out, kcache, vcache, tables, run_start, seq_start)
@@ -1232,11 +1245,12 @@ def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_st
     _need(q.shape[1] >= nh * d and out.shape[1] >= nh * dv, "attention rows are too short for the head layout")
     B, E = _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P)
     _f32(head_scale, "head_scale", nh)
+    _f32(dist_slope, "dist_slope", nh)
     _i32(run_start, "run_start", num_seqs + 1)
     _i32(seq_start, "seq_start", num_seqs)
     _i32(tables, "tables")
     _call("kvcm_attention_window_pool_tiles", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache), _ptr(pk),
-          _ptr(pv), _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), _ptr(head_scale), num_seqs, max_run, nh, nkv,
+          _ptr(pv), _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), _ptr(head_scale), _ptr(dist_slope), num_seqs, max_run, nh, nkv,
           d, dv, B, float(scale), int(window), int(P), E, int(keep_first), float(softcap or 0.0), _stream())
 
 
@@ -1400,24 +1414,139 @@ def softcap_rows(x, cap):
     return x
 
 
-def head_gate(o, gate, heads, dv, rows=None):
-    """o[r, h, :] *= sigmoid(gate[r, h]) in place; o [T, >= heads*dv] in the compute dtype, gate float32 rows of >= heads."""
+def head_gate(o, gate, heads, dv, rows=None, per_element=False):
+    """o[r, h, :] *= sigmoid(gate[r, h]) in place; o [T, >= heads*dv] in the compute dtype, gate float32 rows of >= heads.
+    ``per_element``: a gate logit for every element, o[r, c] *= sigmoid(gate[r, c]), gate rows of >= heads*dv."""
     T = o.shape[0] if rows is None else rows
     _rows2d(o, "o")
-    _f32rows(gate, "gate", heads)
+    _f32rows(gate, "gate", heads * dv if per_element else heads)
     _need(o.is_cuda and o.shape[1] >= heads * dv and gate.shape[0] >= T and o.shape[0] >= T, "head_gate: shapes do not agree")
-    _call("kvcm_head_gate", _ptr(o), _DT[o.dtype], o.stride(0), _ptr(gate), gate.stride(0), T, heads, dv, _stream())
+    _call("kvcm_head_gate", _ptr(o), _DT[o.dtype], o.stride(0), _ptr(gate), gate.stride(0), T, heads, dv, 1 if per_element else 0, _stream())
     return o
 
 
-def rms_groups(x, col0, size, groups, weight, eps, rows=None):
-    """In place on float32 rows: each of ``groups`` stretches of ``size`` columns from col0 on is divided by its root mean
-    square (eps inside the root) and multiplied by weight[0 .. size)."""
+def rms_groups(x, col0, size, groups, weight, eps, rows=None, out=None):
+    """On float32 rows: each of ``groups`` stretches of ``size`` columns from col0 on is divided by its root mean
+    square (eps inside the root) and multiplied by weight[0 .. size); in place, or with ``out`` (rows of any dtype the
+    kernels store, >= groups*size columns) into out from its column 0 on, x left as it is."""
     T = x.shape[0] if rows is None else rows
     _f32rows(x, "x", col0 + size * groups)
     _f32(weight, "weight", size)
-    _call("kvcm_rms_groups", _ptr(x), x.stride(0), col0, size, groups, _ptr(weight), float(eps), T, _stream())
-    return x
+    if out is not None:
+        _rows2d(out, "out")
+        _need(out.is_cuda and out.shape[0] >= T and out.shape[1] >= size * groups, "rms_groups: the output is too small")
+    _call("kvcm_rms_groups", _ptr(x), x.stride(0), col0, size, groups, _ptr(weight), float(eps), _ptr(out),
+          _DT[out.dtype] if out is not None else 0, out.stride(0) if out is not None else 0, T, _stream())
+    return x if out is None else out
+
+
+class BiasedOutput:
+    """A sublayer's output with a bias of its output projection still to be added: ``value`` (a 32-bit tensor or
+    PartialSums) + bias[H].  A norm that adds the sublayer's output to the stream adds the bias in the same pass
+    (``layernorm_post``); anyone else calls ``materialize()``."""
+
+    def __init__(self, value, bias):
+        self.value, self.bias = value, bias
+
+    def materialize(self):
+        out = self.value.materialize() if hasattr(self.value, "materialize") else self.value
+        out += self.bias      # (a tensor library's routine: not for recorded steps)
+        return out
+
+
+def layernorm_post(x, weight, eps, alpha=1.0, add=None, out=None, rows=None):
+    """x <- ln(alpha * x + add) * weight in place, ln(v) = (v - mean) / sqrt(mean of squared deviations + eps), all in
+    32-bit; ``add``: a 32-bit tensor like x, PartialSums, a BiasedOutput of either, or None.  ``out`` [R, H] also receives
+    the new rows, rounded once to its dtype.  With ``rows`` (int32 [R]) the result of those rows goes to ``out`` only."""
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.is_cuda and x.dim() == 2, "x must be contiguous float32 [T, H]")
+    T, H = x.shape
+    _f32(weight, "the norm weight", H)
+    bias, a, splits = None, None, 1
+    if isinstance(add, BiasedOutput):
+        add, bias = add.value, add.bias
+        _f32(bias, "the output bias", H)
+    if isinstance(add, PartialSums):
+        _need(add.rows == T and add.cols == H, "the added product's partial sums must match x")
+        a, splits = add.data, add.splits
+    elif add is not None:
+        _need(add.dtype == torch.float32 and add.is_contiguous() and add.shape == x.shape and add.is_cuda, "the added output must match x")
+        a = add
+    R = T
+    if out is not None:
+        _need(out.is_cuda and out.is_contiguous() and out.dim() == 2 and out.shape[1] == H, "out must be contiguous [R, H]")
+        R = out.shape[0]
+        if rows is not None:
+            _i32(rows, "rows", R)
+        else:
+            _need(R <= T, "x has fewer rows than the output")
+    else:
+        _need(rows is None, "layernorm_post: gathered rows need an output")
+    _call("kvcm_layernorm_post", _ptr(x), _ptr(a), splits, T * H, _ptr(bias), float(alpha), _ptr(weight), _ptr(rows), _ptr(out),
+          _DT[out.dtype] if out is not None else 0, R, H, float(eps), _stream())
+    return out
+
+
+def head_norm_store(qkv, q_out, nh, nkv, d, dv, eps, q_weight=None, k_weight=None, bias=None, positions=None, temp_coef=0.0,
+                    temp_every=0, values_are_keys=False, slots=None, kcache=None, vcache=None, rows=None):
+    """qkv: 32-bit rows [q (nh*d) | k (nkv*d) | v (nkv*dv)] (no v with ``values_are_keys``); ``bias``: a float32 row of
+    that layout, added first.  Every q and k head is divided by its own root mean square (eps inside the root) and
+    multiplied by ``q_weight`` / ``k_weight`` [d] (None: that kind passes); with ``temp_every`` > 0 the query is then
+    multiplied by 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1).  q goes to q_out [T, nh*d], k to its page
+    slot, and as values the projection's own or, with ``values_are_keys``, the keys as projected, before their norm."""
+    T = q_out.shape[0] if rows is None else rows
+    width = (nh + nkv) * d + (0 if values_are_keys else nkv * dv)
+    _f32rows(qkv, "qkv", width)
+    _rows2d(q_out, "q_out")
+    _need(q_out.shape[1] >= nh * d and q_out.is_cuda and qkv.shape[0] >= T, "head_norm_store: shapes do not agree")
+    _need(not values_are_keys or d == dv, "head_norm_store: keys can only be values of their own size")
+    _f32(q_weight, "q_weight", d)
+    _f32(k_weight, "k_weight", d)
+    _f32(bias, "bias", width)
+    if temp_every > 0:
+        _i32(positions, "positions", T)
+        _need(positions is not None, "head_norm_store: a temperature by position needs the positions")
+    B = 1
+    if slots is not None:
+        _i32(slots, "slots", T)
+        _need(kcache is not None and kcache.dtype == q_out.dtype and kcache.is_contiguous() and kcache.dim() == 4
+              and kcache.shape[1] == nkv and kcache.shape[3] == d, "key cache must be [pages, nkv, block_size, d]")
+        B = kcache.shape[2]
+        _need(vcache is not None and vcache.dtype == q_out.dtype and vcache.is_contiguous()
+              and tuple(vcache.shape) == (kcache.shape[0], nkv, dv, B), "value cache must be [pages, nkv, dv, block_size]")
+    _call("kvcm_head_norm_store", _ptr(qkv), qkv.stride(0), _ptr(bias), _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(positions),
+          float(temp_coef), int(temp_every), 1 if values_are_keys else 0, _ptr(slots), _ptr(q_out), _DT[q_out.dtype], q_out.stride(0),
+          _ptr(kcache), _ptr(vcache), T, nh, nkv, d, dv, B, _stream())
+
+
+def gemm_heads(x, w, out, gate=None, rows=None):
+    """out[m, h*N + n] = sum_k x[m, h*K + k] * w[h, n, k] for w [heads, N, K]: one small product per head, every head on
+    its own stretch of the rows.  x and w in one dtype (float32 gives float32); ``gate`` (float32 rows of >= heads*N):
+    the result times sigmoid(gate), element by element, before it is stored."""
+    _dev(x, w, out, gate)
+    _rows2d(x, "x")
+    _rows2d(out, "out")
+    _need(w.dim() == 3 and w.is_contiguous() and w.dtype == x.dtype, "gemm_heads: w must be contiguous [heads, N, K] in x's dtype")
+    heads, N, K = w.shape
+    M = out.shape[0] if rows is None else rows
+    _need(x.shape[0] >= M and x.shape[1] >= heads * K and out.shape[1] >= heads * N, "gemm_heads: shapes do not agree")
+    _need(x.dtype != torch.float32 or out.dtype == torch.float32, "gemm_heads: float32 operands give a float32 result")
+    if gate is not None:
+        _f32rows(gate, "gate", heads * N)
+        _need(gate.shape[0] >= M, "gemm_heads: the gate has fewer rows than the step")
+    _call("kvcm_gemm_heads", _ptr(x), _DT[x.dtype], x.stride(0), _ptr(w), _ptr(out), _DT[out.dtype], out.stride(0), _ptr(gate),
+          gate.stride(0) if gate is not None else 0, M, heads, N, K, _stream())
+    return out
+
+
+def act_rows(x, out, activation):
+    """out[T, I] = act(x[T, :I]) for 32-bit rows; act: "silu", "relu" or "gelu_tanh"."""
+    T, I = out.shape
+    _f32rows(x, "x", I)
+    _rows2d(out, "out")
+    _need(x.shape[0] >= T and out.is_cuda, "act_rows: the rows do not agree")
+    _need(activation in GATE_ACTIVATIONS, f"unknown activation {activation!r} ({sorted(GATE_ACTIVATIONS)})")
+    _call("kvcm_act_rows", _ptr(x), x.stride(0), _ptr(out), _DT[out.dtype], out.stride(0), T, I, GATE_ACTIVATIONS[activation], _stream())
+    return out
 
 
 def mlstm_scan(q, k, v, gate_in, gate_keep, in_bias, keep_bias, cap, q_scale, coef, n_new, o, s_state, n_state, m_state, step, heads, dk, dv):
@@ -1442,16 +1571,17 @@ def mlstm_scan(q, k, v, gate_in, gate_keep, in_bias, keep_bias, cap, q_scale, co
     return o
 
 
-def moe_route(logits, experts, top, chosen, weight, rows=None):
+def moe_route(logits, experts, top, chosen, weight, rows=None, over_chosen=False):
     """chosen[T, top] (int32) and weight[T, top] (float32): the ``top`` experts with the largest softmax scores over all
-    ``experts`` of each row's 32-bit router logits, best first, with those scores."""
+    ``experts`` of each row's 32-bit router logits, best first, with those scores; ``over_chosen``: with the softmax over
+    the chosen logits alone instead (the weights of a row add up to one)."""
     T = chosen.shape[0] if rows is None else rows
     _f32rows(logits, "logits", experts)
     _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.is_cuda and chosen.shape[1] == top and chosen.shape[0] >= T,
           "chosen must be int32 [T, top]")
     _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.is_cuda and tuple(weight.shape) == tuple(chosen.shape),
           "weight must be float32 [T, top]")
-    _call("kvcm_moe_route", _ptr(logits), logits.stride(0), experts, top, _ptr(chosen), _ptr(weight), T, _stream())
+    _call("kvcm_moe_route", _ptr(logits), logits.stride(0), experts, top, 1 if over_chosen else 0, _ptr(chosen), _ptr(weight), T, _stream())
 
 
 def moe_table_route(tokens, table, top, chosen, weight, rows=None):

@@ -58,7 +58,8 @@ class ParamSpec:
     """A tensor a part wants.  ``sources`` are (checkpoint name, shape) pairs concatenated along
     dim 0 in that order (one pair = taken as it is).  ``role`` decides the stored precision:
       matrix / table  the compute dtype (bfloat16 when serving, float32 in the 32-bit path)
-      vector          as stored when that is 32-bit, else the compute dtype
+      vector          as stored when that is 32-bit, else the compute dtype (a norm's weight: random weights lie around 1)
+      bias            stored like a vector; random weights lie around 0
       index           integer tables, kept as int32.
     ``distinct_below`` (index tables): what valid entries look like, for whoever makes random ones: every row holds
     distinct values in [0, distinct_below) (0: any values)."""

@@ -167,3 +167,24 @@ class GatedFeedForward(FeedForward):
             gu = linear32(self.ctx, step, h, self.w["w_gate_up"], "gated_gate_up")
             ops.gated_act(gu, act, kind)
         return linear32(self.ctx, step, act, self.w["w_down"], "gated_out")
+
+
+@FEED_FORWARDS.register("plain_mlp")
+class PlainFeedForward(FeedForward):
+    """down(act(up(h))): a feed-forward without a gate; the first product's 32-bit sums go straight into the activation.
+    params: intermediate_size, activation ("relu" | "silu" | "gelu_tanh"); up, down: the checkpoint names after the
+    prefix (defaults "up", "down").  The result is 32-bit: a norm reads it."""
+
+    capturable = True
+
+    def param_specs(self):
+        H, I, pre, p = self.ctx.hidden_size, self.params["intermediate_size"], self.prefix, self.params
+        return [ParamSpec("w_up", ((pre + p.get("up", "up"), (I, H)),)),
+                ParamSpec("w_down", ((pre + p.get("down", "down"), (H, I)),))]
+
+    def forward(self, step, h):
+        I, ops = self.params["intermediate_size"], self.ctx.ops
+        up = linear32(self.ctx, step, h, self.w["w_up"], "plain_up")
+        act = step.ws("plain_act", (step.rows, I))
+        ops.act_rows(up, act, self.params.get("activation", "gelu_tanh"))
+        return linear32(self.ctx, step, act, self.w["w_down"], "plain_out", keep_partial=True)      # the stream's next norm adds the slices

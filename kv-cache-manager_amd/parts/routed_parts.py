@@ -23,6 +23,7 @@ class RoutedExperts(FeedForward):
     """Which experts a row uses (``routing``):
       "softmax" (default)  router logits z = W_router h in 32-bit, scores s = softmax(z) over all experts; the ``top``
                            experts with the largest scores, weighted by their scores as they are (not renormalized)
+      "softmax_chosen"     the ``top`` experts with the largest logits, weighted by the softmax over those logits alone
       "table"              an integer table [vocabulary, top] names the experts of every token id; each weighs 1 / top
     What an expert computes (``activation``):
       "relu2" (default)    W_down act(W_up h), act = the square of relu
@@ -40,8 +41,8 @@ class RoutedExperts(FeedForward):
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
         self.routing, self.activation = params.get("routing", "softmax"), params.get("activation", "relu2")
-        if self.routing not in ("softmax", "table"):
-            raise ValueError(f"routed_experts {prefix!r}: routing {self.routing!r} is not supported (softmax | table)")
+        if self.routing not in ("softmax", "softmax_chosen", "table"):
+            raise ValueError(f"routed_experts {prefix!r}: routing {self.routing!r} is not supported (softmax | softmax_chosen | table)")
         if self.activation not in ("relu2", "silu_gated"):
             raise ValueError(f"routed_experts {prefix!r}: activation {self.activation!r} is not supported (relu2 | silu_gated)")
         self.gated = self.activation == "silu_gated"
@@ -113,7 +114,7 @@ class RoutedExperts(FeedForward):
             ops.moe_table_route(step.tokens, w["table"], top, chosen, weight, rows=T)
         else:
             logits = linear32(self.ctx, step, h, w["w_router"], "routed_logits")
-            ops.moe_route(logits, E, top, chosen, weight, rows=T)
+            ops.moe_route(logits, E, top, chosen, weight, rows=T, over_chosen=self.routing == "softmax_chosen")
         add = self.shared.forward(step, h) if self.shared is not None else None      # 32-bit [T, H]: the experts' sum starts from it
         H = self.ctx.hidden_size
         act = step.ws("routed_act", (T, top * F)).view(T * top, F)

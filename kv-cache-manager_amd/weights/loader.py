@@ -7,8 +7,8 @@ move data.  The reference fuses q/k/v and gate/up in its exporter (tools/export_
 and has no by-name loading; the fusing here happens at load time on the device.
 
 Stored precision: matrices and tables take the compute dtype (bfloat16 when serving, float32 in
-the 32-bit path); a vector that the checkpoint stores in 32 bits stays 32-bit; integer tables
-become int32.
+the 32-bit path); a vector (a norm's weight, a bias) that the checkpoint stores in 32 bits stays
+32-bit; integer tables become int32.
 """
 import json
 import os
@@ -79,7 +79,7 @@ def _stored_dtype(role, stored: torch.dtype, compute: torch.dtype) -> torch.dtyp
         raise WeightsError("a floating-point tensor is stored as integers")
     if compute == torch.float32:
         return torch.float32
-    if role == "vector" and stored in (torch.float32, torch.float64):
+    if role in ("vector", "bias") and stored in (torch.float32, torch.float64):
         return torch.float32
     return compute
 

@@ -86,7 +86,7 @@ def _distinct_rows(raw: torch.Tensor, below: int) -> torch.Tensor:
 
 def random_tensor(seed: int, name: str, shape, role: str, dtype=torch.bfloat16, std=0.02, norm_jitter=0.0, device="cpu",
                   distinct_below=0):
-    """One tensor of the rule.  role "vector": 1 + norm_jitter * n; "index": int32 in [0, INDEX_MODULUS), or with
+    """One tensor of the rule.  role "vector": 1 + norm_jitter * n; "bias": std * n like a matrix; "index": int32 in [0, INDEX_MODULUS), or with
     ``distinct_below`` rows of distinct values below that; else std * n.  On a GPU the fill kernel makes the values in place."""
     if any(n < 0 for n in shape):
         raise ValueError(f"{name}: a size of this tensor is left to the checkpoint ({tuple(shape)}); random weights need it in "
