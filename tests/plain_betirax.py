@@ -157,7 +157,7 @@ def window_attention(h, w, pre, m, eps, positions=None):
 
 def latent_kv(h, w, pre, m, eps, positions):
     """-> (latent c [T, kv_rank], the rotated key part shared by all heads [T, rot_dim]): what a request keeps."""
-    r, rd = m["kv_rank"], m["rot_dim"]
+    r, rd = m["kv_rank"], m.get("rot_dim", 0)
     dkv = h @ w[pre + "dkv"].T
     c = rms(dkv[:, :r], eps) * w[pre + "dkv.norm"]
     rot = m.get("rot") or {}
@@ -171,7 +171,7 @@ def latent_attention(h, w, pre, m, eps, kv=None, positions=None):
     """The mixer 'latent_attention'.  ``kv``: another layer's (c, rotated key part), for a layer without W_dkv."""
     T = h.shape[0]
     positions = np.arange(T) if positions is None else positions
-    H, d, rd, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+    H, d, rd, dv = m["heads"], m["dim"], m.get("rot_dim", 0), m.get("vdim", m["dim"])
     cq = rms(h @ w[pre + "dq"].T, eps) * w[pre + "dq.norm"]
     q = (cq @ w[pre + "uq"].T).reshape(T, H, d + rd)
     c, kr = latent_kv(h, w, pre, m, eps, positions) if kv is None else kv
@@ -226,7 +226,7 @@ def feed_forward(h, w, pre, mlp):
 # ------------------------------------------------------------------------------------ model
 def forward(raw, w, tokens, trace=None):
     """Logits [T, vocab] of one sequence.  ``trace``: a list that receives the stream after every layer."""
-    eps, alpha = raw["norm"]["eps"], raw["postln_alpha"]
+    eps, alpha = raw["norm"]["eps"], raw.get("postln_alpha", 1.0)
     tokens = np.asarray(tokens)
     x = w["embed"][tokens] * (raw.get("embedding") or {}).get("scale", 1.0)
     kept = {}
