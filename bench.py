@@ -3,7 +3,7 @@
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512] [--layers L]
                   [--sizes tinyllama-1.1b|llama-2-7b|llama-3-8b] [--context-limit 2048] [--prefill-tokens 2048]
                   [--tune-products off|heuristic|all] [--no-points] [--only-prefill]
-  python bench.py --design kasuvik|furapel|fisesun [--design-sizes 2048,4096] [--layers 4] [--prefill-tokens 2048] [--steps K]
+  python bench.py --design kasuvik|furapel|fisesun|betirax [--design-sizes 2048,4096] [--layers 4] [--prefill-tokens 2048] [--steps K]
 
 A "step" is one decode step of the whole engine (schedule, batch metadata, upload, model step on
 the GPU, sampling, download, update).  W untimed steps, then exactly K timed steps between two
@@ -22,6 +22,11 @@ and the Llama decoder at equal width, heads, active feed-forward width and depth
 --design fisesun does the same for the Fisesun decoder (layers that norm a sublayer's output only: grouped-query attention
 with q and k normed over the whole projection, capped scores, a window that keeps the first tokens, blended values; a
 matrix memory; gated experts named by a table per token id beside a shared expert) beside the Furapel and the Llama decoder.
+
+--design betirax does the same for the Betirax decoder (layers that norm after the sum: grouped-query attention with a norm
+per head, keys as values, a query temperature, a distance bias, a window and a gate per element; latent attention with a
+rotated key part and query latents; a dense feed-forward or gated experts weighted over the chosen logits beside a shared
+expert) beside the Fisesun and the Llama decoder.
 """
 import argparse
 import json
@@ -216,6 +221,40 @@ def fisesun_config(width, layers, vocab=32000):
                                     "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "layers": listed})
 
 
+# Betirax at a width: (cached latent, rotated key part, query latent, positions per temperature step, experts, experts a row)
+BETIRAX_SIZES = {2048: (96, 32, 768, 1024, 8, 2), 4096: (96, 32, 1536, 1024, 8, 2)}
+
+
+def betirax_config(width, layers, vocab=32000):
+    """A Betirax configuration at a width of DESIGN_SIZES: layers attention, attention, latent attention, attention in turn
+    (every second latent attention reads the pages of the one before it); the first and third of four are followed by a
+    dense feed-forward, the others by ``experts`` gated experts of which a row uses ``top`` and a shared expert (the ``top``
+    experts a quarter each and the shared one half of the dense feed-forward's width)."""
+    from kvcm_amd.config.betirax_config import BetiraxConfig
+    nh, nkv, hd, ff, window = DESIGN_SIZES[width][:5]
+    rank, rot, q_rank, every, experts, top = BETIRAX_SIZES[width]
+    moe = {"kind": "moe", "expert": {"ff": ff // (2 * top)}, "router": {"experts": experts, "top": top}, "shared": {"ff": ff // 2}}
+    dense = {"kind": "dense", "ff": ff}
+    attention = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": window},
+                 "q_temp": {"coef": 0.5, "every": every}}
+    latent = {"heads": nh, "dim": hd, "rot_dim": rot, "vdim": hd, "kv_rank": rank, "q_rank": q_rank, "scale": (hd + rot) ** -0.5,
+              "rot": {"dims": rot, "base": 10000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    listed, owner = [], None
+    for i in range(layers):
+        mlp = dense if i % 2 == 0 else moe
+        if i % 4 == 2:
+            mixer = dict(latent)
+            if owner is not None:
+                mixer["kv_from"], owner = owner, None
+            else:
+                owner = i
+            listed.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
+        else:
+            listed.append({"type": "attention", "mixer": attention, "mlp": mlp})
+    return BetiraxConfig.from_dict({"architecture": "Betirax", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+                                    "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "layers": listed})
+
+
 def design_main(args):
     import torch
     from kvcm_amd.config.engine_config import EngineConfig
@@ -230,7 +269,7 @@ def design_main(args):
     first = args.design
     record = {"metric": "prefill and decode tok/s of the %s decoder beside the %s at equal sizes"
                         % (first.capitalize(), {"kasuvik": "Llama decoder", "furapel": "Kasuvik and Llama decoders",
-                                                 "fisesun": "Furapel and Llama decoders"}[first]), "dtype": key,
+                                                 "fisesun": "Furapel and Llama decoders", "betirax": "Fisesun and Llama decoders"}[first]), "dtype": key,
               "data": "synthetic", "layers": layers, "prefill_tokens": T, "prompt_len": args.prompt_len, "steps": steps, "sizes": {}}
     for width in [int(w) for w in args.design_sizes.split(",")]:
         if width not in DESIGN_SIZES:
@@ -242,10 +281,12 @@ def design_main(args):
             designs = {"furapel": furapel_config(width, layers), **designs}
         elif first == "fisesun":
             designs = {"fisesun": fisesun_config(width, layers), "furapel": furapel_config(width, layers), "llama": designs["llama"]}
+        elif first == "betirax":
+            designs = {"betirax": betirax_config(width, layers), "fisesun": fisesun_config(width, layers), "llama": designs["llama"]}
         if args.design_alone:
             designs = {first: designs[first]}
         for name, cfg in designs.items():
-            arch = {"kasuvik": "Kasuvik", "furapel": "Furapel", "fisesun": "Fisesun", "llama": "LlamaForCausalLM"}[name]
+            arch = {"kasuvik": "Kasuvik", "furapel": "Furapel", "fisesun": "Fisesun", "betirax": "Betirax", "llama": "LlamaForCausalLM"}[name]
             tensors = random_tensors(arch, cfg, seed=0, dtype=dt, device="cuda:0")
             ec = EngineConfig(block_size=16, max_seq_len=limit, num_blocks=8 * limit // 16, max_num_seqs=8,
                               max_batched_tokens=max(4096, T + 64), dtype=args.dtype, max_logit_rows=64, beyond_max_position=True)
@@ -298,10 +339,11 @@ def main():
                     help="run nothing but the 2,048-token prefill (for a profiler); prints its record alone")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="tokens of the prefill measurement (2,048 in the record; other lengths for sweeps)")
-    ap.add_argument("--design", default="llama", choices=["llama", "kasuvik", "furapel", "fisesun"],
+    ap.add_argument("--design", default="llama", choices=["llama", "kasuvik", "furapel", "fisesun", "betirax"],
                     help="llama: the workload above (the default); kasuvik: prefill and decode of the Kasuvik decoder beside the "
                          "Llama decoder at equal sizes; furapel: the same for the Furapel decoder beside both; "
-                         "fisesun: the same for the Fisesun decoder beside the Furapel and the Llama decoder "
+                         "fisesun: the same for the Fisesun decoder beside the Furapel and the Llama decoder; "
+                         "betirax: the same for the Betirax decoder beside the Fisesun and the Llama decoder "
                          "(--design-sizes, --layers, --prefill-tokens, --prompt-len, --steps)")
     ap.add_argument("--design-sizes", default="2048,4096", help="widths of the --design comparison (2048, 4096)")
     ap.add_argument("--design-alone", action="store_true", help="run the --design itself only, not the designs beside it (for a profiler)")
