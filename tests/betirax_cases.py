@@ -5,7 +5,8 @@ multiples of 16, one expert, as many experts a token as there are, one head, as 
 for all, a rotated key part that is absent, partly and wholly rotated, with and without rescaling, latent sizes that the
 matrix-core kernels take and sizes that they refuse, windows of one token, shorter and longer than a page and none,
 query temperatures whose steps are shorter and longer than a page and none, a stream factor of one (left out of the
-file) and others, and layers that read an earlier layer's pages right after it and several layers later.
+file) and others, and layers that read an earlier layer's pages right after it and several layers later, two of them the
+same layer's.
 """
 import numpy as np
 import torch
@@ -71,7 +72,8 @@ CONFIGS = {
           "layers": [_layer(_attention(1, 1, 10, 0.35, window=1), _moe(1, 1, 12)),
                      _layer(_latent(1, 6, 0, 10, 7, 5, 0.4), _moe(2, 2, 8, shared=8)),
                      _layer(_attention(3, 3, 16, 0.3, window=40, temp=(1.0, 1)), None),
-                     _layer(_latent(2, 16, 0, 8, 7, 9, 0.3, kv_from=1), _dense(24))]},
+                     _layer(_latent(2, 16, 0, 8, 7, 9, 0.3, kv_from=1), _dense(24)),
+                     _layer(_latent(3, 4, 0, 12, 7, 11, 0.5, kv_from=1), _moe(3, 2, 16))]},
     # pages of 32, 128-wide heads with three query heads per KV head, a long window, a wholly rotated key part without rescaling
     "S": {"architecture": "Betirax", "vocab": 200, "width": 96, "embedding": {"scale": 0.5}, "norm": {"eps": 1e-5}, "postln_alpha": 3.0,
           "layers": [_layer(_attention(6, 2, 128, 0.09, window=70, temp=(0.25, 64)), _moe(8, 3, 48, shared=64)),
