@@ -7,7 +7,8 @@
 //                            tokens j < keep_first (the sequence's first tokens stay visible beyond the window)
 //   and all of them share one softmax; score = (q . k) * scale_h with a factor per query head, and with a cap c > 0
 //   score <- c tanh(score / c); then, with a slope per query head, score <- score - slope_h * (i - j) for token j (a bias
-//   that grows with the distance; not offered together with pooled blocks, which have no one distance).
+//   that grows with the distance; not offered together with pooled blocks, which have no one distance).  The output may be
+//   multiplied element by element with sigmoid(gate) (32-bit gate logits of the output's shape) before it is stored.
 //
 // Pages: keys [pages, kv_heads, B, d], values transposed [pages, kv_heads, dv, B] (as the other
 // attentions of this library keep them).  Pooled entries are 32-bit and live with the page that holds
@@ -70,7 +71,17 @@ __global__ void __launch_bounds__(256)
   const float2* cs = cos_sin + size_t(row) * (rot / 2);
   const int slot = slots ? slots[row] : -1;
   const int heads = slot >= 0 ? nh + nkv : nh;
-  for (int e = threadIdx.x; e < heads * d; e += blockDim.x) {
+  // grid (rows, 1): one workgroup does a whole row; grid (rows, nh + nkv + 1), for steps of few rows: workgroup y does
+  // head y of q | k and the last one the values (the same operations on every element either way)
+  int e0 = 0, e1 = heads * d;
+  bool values = true;
+  if (gridDim.y > 1) {
+    const int part = blockIdx.y;
+    values = part == nh + nkv;
+    e0 = values || part >= heads ? 0 : part * d;
+    e1 = values || part >= heads ? 0 : e0 + d;
+  }
+  for (int e = e0 + threadIdx.x; e < e1; e += blockDim.x) {
     const int head = e / d, i = e % d;
     const float* r = head < nh ? rq + size_t(head) * d : rk + size_t(head - nh) * d;      // this head's entries
     float x = r[i];
@@ -84,7 +95,7 @@ __global__ void __launch_bounds__(256)
     if (head < nh) store_f(q_out + size_t(row) * ldq + e, x);
     else if (slot >= 0) store_f(kcache + ((size_t(slot / B) * nkv + (head - nh)) * B + slot % B) * d + i, x);
   }
-  if (slot < 0) return;
+  if (slot < 0 || !values) return;
   const float* v = rk + size_t(nkv) * d;
   for (int e = threadIdx.x; e < nkv * dv; e += blockDim.x) {
     const int head = e / dv, i = e % dv;
@@ -252,7 +263,7 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
                                  const float* __restrict__ pk, const float* __restrict__ pv,
                                  const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
                                  const int* __restrict__ ctx_lens, const float* __restrict__ head_scale,
-                                 const float* __restrict__ dist_slope,
+                                 const float* __restrict__ dist_slope, const float* __restrict__ gate, int ldg,
                                  int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E, int keep_first,
                                  float softcap) {
   extern __shared__ float lds[];      // [d] q * scale * head_scale[h]; [waves][64] probabilities; [waves][dv + 2] results
@@ -411,7 +422,9 @@ __global__ void __launch_bounds__(kWpWaves* kWave)
     float acc = 0.f;
 #pragma unroll
     for (int w = 0; w < kWpWaves; ++w) acc = fmaf(merge[w * (dv + 2) + cc], wgt[w], acc);
-    store_f(orow + cc, acc / ll);
+    float res = acc / ll;
+    if (gate) res *= 1.0f / (1.0f + expf(-gate[size_t(row) * ldg + size_t(head) * dv + cc]));      // a gate per element of the output
+    store_f(orow + cc, res);
   }
 }
 
@@ -453,11 +466,12 @@ int kvcm_rotate_store(const float* src, int ld, const float* kv_src, int ldkv, c
   else KVCM_REQUIRE(ld >= (slots ? (nh + nkv) * d + nkv * dv : nh * d) && ldq >= nh * d, "rotate_store: row strides too small");
   KVCM_REQUIRE(!slots || (kcache && vcache), "rotate_store: slots without pages");
   const float2* cs = reinterpret_cast<const float2*>(cos_sin);
+  const dim3 T_by_parts(T, T <= kNormRotateFewRows ? nh + nkv + 1 : 1);
   if (dtype == kF32)
-    rotate_store_kernel<float><<<T, 256, 0, s>>>(src, ld, kv_src, ldkv, cs, rot, halves, slots, static_cast<float*>(q_out), ldq,
+    rotate_store_kernel<float><<<T_by_parts, 256, 0, s>>>(src, ld, kv_src, ldkv, cs, rot, halves, slots, static_cast<float*>(q_out), ldq,
                                                   static_cast<float*>(kcache), static_cast<float*>(vcache), nh, nkv, d, dv, B);
   else if (dtype == kBF16)
-    rotate_store_kernel<bf16_t><<<T, 256, 0, s>>>(src, ld, kv_src, ldkv, cs, rot, halves, slots, static_cast<bf16_t*>(q_out), ldq,
+    rotate_store_kernel<bf16_t><<<T_by_parts, 256, 0, s>>>(src, ld, kv_src, ldkv, cs, rot, halves, slots, static_cast<bf16_t*>(q_out), ldq,
                                                    static_cast<bf16_t*>(kcache), static_cast<bf16_t*>(vcache), nh, nkv, d, dv, B);
   else KVCM_REQUIRE(false, "rotate_store: unknown dtype %d", dtype);
   return launch_status("rotate_store");
@@ -510,9 +524,9 @@ int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* p
 
 int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
-                               const int* ctx_lens, const float* head_scale, const float* dist_slope, int T, int nh, int nkv,
-                               int d, int dv, int B, float scale, int window, int P, int E, int keep_first, float softcap,
-                               hipStream_t s) {
+                               const int* ctx_lens, const float* head_scale, const float* dist_slope, const float* gate, int ldg,
+                               int T, int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E, int keep_first,
+                               float softcap, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && nh > 0 && nkv > 0 && B > 0 && d > 0, "attention_window_pool: bad sizes T=%d heads=%d kv_heads=%d", T, nh, nkv);
   KVCM_REQUIRE(nh % nkv == 0, "attention_window_pool: %d query heads are not a multiple of %d kv heads", nh, nkv);
@@ -523,19 +537,20 @@ int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int
   KVCM_REQUIRE(P == 0 || (pk && pv && E == (B + P - 1) / P), "attention_window_pool: pooled blocks need their entries");
   KVCM_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attention_window_pool: negative count of kept tokens or score cap");
   KVCM_REQUIRE(!dist_slope || P == 0, "attention_window_pool: a distance bias beside pooled blocks is not supported");
+  KVCM_REQUIRE(!gate || ldg >= nh * dv, "attention_window_pool: the gate's rows are too short");
   const long long blocks = static_cast<long long>(T) * nh;
   KVCM_REQUIRE(blocks < (1ll << 31), "attention_window_pool: too many rows");
   const size_t lds = sizeof(float) * (d + kWpWaves * kWave + kWpWaves * (dv + 2));
   if (dtype == kF32)
     attention_window_pool_kernel<float><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
         static_cast<const float*>(q), ldq, static_cast<float*>(out), ldo, static_cast<const float*>(kcache),
-        static_cast<const float*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, dist_slope, nh,
-        nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
+        static_cast<const float*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, dist_slope, gate,
+        ldg, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   else if (dtype == kBF16)
     attention_window_pool_kernel<bf16_t><<<static_cast<unsigned>(blocks), kWpWaves * kWave, lds, s>>>(
         static_cast<const bf16_t*>(q), ldq, static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(kcache),
-        static_cast<const bf16_t*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, dist_slope, nh,
-        nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
+        static_cast<const bf16_t*>(vcache), pk, pv, tables, table_stride, row_seq, ctx_lens, head_scale, dist_slope, gate,
+        ldg, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   else KVCM_REQUIRE(false, "attention_window_pool: unknown dtype %d", dtype);
   return launch_status("attention_window_pool");
 }

@@ -9,7 +9,8 @@
 // costs them nothing but zeros; a row's chunks and their order depend on its own position only.  The first
 // keep_first tokens of a sequence may stay visible beyond the window (chunks of their own, from token 0), and the
 // scores may be capped, score <- c tanh(score / c), and a bias that grows with the distance may be taken off them,
-// score <- score - slope_h * (i - j) with a slope per query head (tokens only: not beside pooled blocks).
+// score <- score - slope_h * (i - j) with a slope per query head (tokens only: not beside pooled blocks); the output may be
+// multiplied element by element with sigmoid(gate) before it is stored.
 // bfloat16 storage only; sizes d and dv in multiples of 8, pages whose size is a multiple of 8 and divides 64.
 #include <cfloat>
 
@@ -36,7 +37,7 @@ __global__ void __launch_bounds__(256)
                                        const float* __restrict__ pk, const float* __restrict__ pv,
                                        const int* __restrict__ tables, int table_stride, const int* __restrict__ run_start,
                                        const int* __restrict__ seq_start, const float* __restrict__ head_scale,
-                                       const float* __restrict__ dist_slope, int tiles_per_seq,
+                                       const float* __restrict__ dist_slope, const float* __restrict__ gate, int ldg, int tiles_per_seq,
                                        int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E,
                                        int keep_first, float softcap) {
   constexpr int KP = DP + 8, KS = DP / 32, DVP = DVT * 16;
@@ -247,7 +248,11 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int vt = 0; vt < DVT; ++vt) {
         const int cc = vt * 16 + col;
-        if (cc < dv) out[size_t(r0 + row) * ldo + size_t(head) * dv + cc] = float_to_bf16_bits(o[vt][i] * inv);
+        if (cc < dv) {
+          float res = o[vt][i] * inv;
+          if (gate) res *= 1.0f / (1.0f + expf(-gate[size_t(r0 + row) * ldg + size_t(head) * dv + cc]));      // a gate per element
+          out[size_t(r0 + row) * ldo + size_t(head) * dv + cc] = float_to_bf16_bits(res);
+        }
       }
     }
   }
@@ -256,11 +261,11 @@ __global__ void __launch_bounds__(256)
 template <int DP>
 int launch_tiles(int dvt, dim3 grid, hipStream_t s, const uint16_t* q, int ldq, uint16_t* out, int ldo, const uint16_t* kc,
                  const uint16_t* vc, const float* pk, const float* pv, const int* tables, int table_stride, const int* run_start,
-                 const int* seq_start, const float* head_scale, const float* dist_slope, int tiles_per_seq, int nh, int nkv, int d,
-                 int dv, int B, float scale, int window, int P, int E, int keep_first, float softcap) {
+                 const int* seq_start, const float* head_scale, const float* dist_slope, const float* gate, int ldg, int tiles_per_seq,
+                 int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E, int keep_first, float softcap) {
 #define KVCM_TILES(DVT)                                                                                                     \
   attention_window_pool_tiles_kernel<DP, DVT><<<grid, 256, 0, s>>>(q, ldq, out, ldo, kc, vc, pk, pv, tables, table_stride,   \
-                                                                   run_start, seq_start, head_scale, dist_slope, tiles_per_seq, \
+                                                                   run_start, seq_start, head_scale, dist_slope, gate, ldg, tiles_per_seq, \
                                                                    nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap)
   if (dvt <= 2) KVCM_TILES(2);
   else if (dvt <= 4) KVCM_TILES(4);
@@ -284,7 +289,7 @@ int kvcm_attention_window_pool_tiles_supported(int d, int dv, int B) {
 int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                      const float* pk, const float* pv, const int* tables, int table_stride,
                                      const int* run_start, const int* seq_start, const float* head_scale, const float* dist_slope,
-                                     int S, int max_run, int nh, int nkv, int d, int dv, int B, float scale, int window, int P,
+                                     const float* gate, int ldg, int S, int max_run, int nh, int nkv, int d, int dv, int B, float scale, int window, int P,
                                      int E, int keep_first, float softcap, hipStream_t s) {
   if (S == 0 || max_run == 0) return 0;
   KVCM_REQUIRE(S > 0 && max_run > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_window_pool_tiles: bad sizes");
@@ -297,6 +302,7 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
   KVCM_REQUIRE(P == 0 || d % 8 == 0, "attention_window_pool_tiles: pooled keys are read eight at a time");
   KVCM_REQUIRE(keep_first >= 0 && softcap >= 0.f, "attention_window_pool_tiles: negative count of kept tokens or score cap");
   KVCM_REQUIRE(!dist_slope || P == 0, "attention_window_pool_tiles: a distance bias beside pooled blocks is not supported");
+  KVCM_REQUIRE(!gate || ldg >= nh * dv, "attention_window_pool_tiles: the gate's rows are too short");
   const int tiles_per_seq = (max_run + kTileRows - 1) / kTileRows;
   KVCM_REQUIRE(static_cast<long long>(S) * tiles_per_seq < (1ll << 31) && nh <= 65535, "attention_window_pool_tiles: too many rows");
   const dim3 grid(S * tiles_per_seq, nh);
@@ -307,12 +313,12 @@ int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo,
   const uint16_t* vc = static_cast<const uint16_t*>(vcache);
   if (d <= 32)
     return launch_tiles<32>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                            dist_slope, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
+                            dist_slope, gate, ldg, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   if (d <= 64)
     return launch_tiles<64>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                            dist_slope, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
+                            dist_slope, gate, ldg, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
   return launch_tiles<128>(dvt, grid, s, qq, ldq, oo, ldo, kc, vc, pk, pv, tables, table_stride, run_start, seq_start, head_scale,
-                           dist_slope, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
+                           dist_slope, gate, ldg, tiles_per_seq, nh, nkv, d, dv, B, scale, window, P, E, keep_first, softcap);
 }
 
 }  // extern "C"

@@ -459,13 +459,17 @@ __global__ void __launch_bounds__(256)
 }
 
 // out[t, i] = act(in[t, i]) for feed-forwards without a gate: the same activations, computed in 32-bit, rounded once.
+// ``in`` may be the un-added slices of a product that was split along K ([splits] arrays, split_stride floats apart): they
+// are added here, in their order.
 template <class TO>
 __global__ void __launch_bounds__(256)
-    act_rows_kernel(const float* __restrict__ in, int ld, TO* __restrict__ out, int ldo, int I, int act) {
+    act_rows_kernel(const float* __restrict__ in, int ld, int splits, size_t split_stride, TO* __restrict__ out, int ldo, int I,
+                    int act) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= I) return;
-  const float g = in[size_t(t) * ld + i];
+  float g = in[size_t(t) * ld + i];
+  for (int sl = 1; sl < splits; ++sl) g += in[size_t(sl) * split_stride + size_t(t) * ld + i];
   float a;
   if (act == 1) a = fmaxf(g, 0.f);
   else if (act == 2) a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
@@ -504,14 +508,17 @@ int kvcm_gated_act(const float* gate_up, int ld, void* out, int out_dtype, int l
   return launch_status("gated_act");
 }
 
-int kvcm_act_rows(const float* in, int ld, void* out, int out_dtype, int ldo, int T, int I, int act, hipStream_t s) {
+int kvcm_act_rows(const float* in, int ld, int splits, long long split_stride, void* out, int out_dtype, int ldo, int T, int I,
+                  int act, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && I > 0 && ld >= I && ldo >= I && in && out, "act_rows: bad sizes T=%d I=%d", T, I);
+  KVCM_REQUIRE(splits >= 1 && split_stride >= 0, "act_rows: an input has at least one slice");
   KVCM_REQUIRE(T <= 65535, "act_rows: too many rows for one launch (%d)", T);
   KVCM_REQUIRE(act >= 0 && act <= 2, "act_rows: unknown activation %d (0 silu, 1 relu, 2 gelu_tanh)", act);
   const dim3 grid((I + 255) / 256, T);
-  if (out_dtype == kF32) act_rows_kernel<float><<<grid, 256, 0, s>>>(in, ld, static_cast<float*>(out), ldo, I, act);
-  else if (out_dtype == kBF16) act_rows_kernel<bf16_t><<<grid, 256, 0, s>>>(in, ld, static_cast<bf16_t*>(out), ldo, I, act);
+  const size_t stride = static_cast<size_t>(split_stride);
+  if (out_dtype == kF32) act_rows_kernel<float><<<grid, 256, 0, s>>>(in, ld, splits, stride, static_cast<float*>(out), ldo, I, act);
+  else if (out_dtype == kBF16) act_rows_kernel<bf16_t><<<grid, 256, 0, s>>>(in, ld, splits, stride, static_cast<bf16_t*>(out), ldo, I, act);
   else KVCM_REQUIRE(false, "act_rows: unknown output dtype %d", out_dtype);
   return launch_status("act_rows");
 }

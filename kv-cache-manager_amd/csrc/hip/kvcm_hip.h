@@ -177,9 +177,9 @@ int kvcm_pool_update(const void* kcache, const void* vcache, int dtype, float* p
                      int dv, int B, int P, int E, hipStream_t s);
 int kvcm_attention_window_pool(const void* q, int dtype, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                const float* pk, const float* pv, const int* tables, int table_stride, const int* row_seq,
-                               const int* ctx_lens, const float* head_scale, const float* dist_slope, int T, int nh, int nkv,
-                               int d, int dv, int B, float scale, int window, int P, int E, int keep_first, float softcap,
-                               hipStream_t s);
+                               const int* ctx_lens, const float* head_scale, const float* dist_slope, const float* gate, int ldg,
+                               int T, int nh, int nkv, int d, int dv, int B, float scale, int window, int P, int E, int keep_first,
+                               float softcap, hipStream_t s);
 // as rotate_store, after q and k were divided by the root mean square of their whole stretch (times a weight) and v was
 // blended with another layer's values of the same row
 int kvcm_norm_rotate_store(const float* src, int ld, const float* wq, const float* wk, float eps, const float* v_other, int ldvo,
@@ -191,7 +191,7 @@ int kvcm_attention_window_pool_tiles_supported(int d, int dv, int B);
 int kvcm_attention_window_pool_tiles(const void* q, int ldq, void* out, int ldo, const void* kcache, const void* vcache,
                                      const float* pk, const float* pv, const int* tables, int table_stride,
                                      const int* run_start, const int* seq_start, const float* head_scale, const float* dist_slope,
-                                     int S, int max_run, int nh, int nkv, int d, int dv, int B, float scale, int window, int P,
+                                     const float* gate, int ldg, int S, int max_run, int nh, int nkv, int d, int dv, int B, float scale, int window, int P,
                                      int E, int keep_first, float softcap, hipStream_t s);
 // (selective_scan.hip, delta_rule.hip) recurrences with a 32-bit state per sequence
 int kvcm_selective_scan(const void* x, int dtype, int ldx, const float* dt_lin, int lddt, const float* dt_bias,
@@ -230,7 +230,8 @@ int kvcm_head_norm_store(const float* src, int ld, const float* bias, const floa
 int kvcm_gemm_heads(const void* X, int in_dtype, int ldx, const void* W, void* Y, int out_dtype, int ldy, const float* gate,
                     int ldg, int M, int heads, int N, int K, hipStream_t s);
 // (elementwise.hip) an activation without a gate on 32-bit rows
-int kvcm_act_rows(const float* in, int ld, void* out, int out_dtype, int ldo, int T, int I, int act, hipStream_t s);
+int kvcm_act_rows(const float* in, int ld, int splits, long long split_stride, void* out, int out_dtype, int ldo, int T, int I,
+                  int act, hipStream_t s);
 // (mlstm.hip) a matrix memory with exponential gates, walked token by token
 int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* ig, int ldi,
                     const float* fg, int ldf, const float* i_bias, const float* f_bias, float cap, float q_scale, float* coef,

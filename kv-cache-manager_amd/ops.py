@@ -108,7 +108,7 @@ def _declare(lib):
     fn("kvcm_layernorm_post", vp, vp, i, C.c_longlong, vp, f, vp, vp, vp, i, i, i, f, vp)
     fn("kvcm_head_norm_store", vp, i, vp, vp, vp, f, vp, f, i, i, vp, vp, i, i, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_gemm_heads", vp, i, i, vp, vp, i, i, vp, i, i, i, i, i, vp)
-    fn("kvcm_act_rows", vp, i, vp, i, i, i, i, i, vp)
+    fn("kvcm_act_rows", vp, i, i, C.c_longlong, vp, i, i, i, i, i, vp)
     fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_moe_route", vp, i, i, i, i, vp, vp, i, vp)
     fn("kvcm_moe_table_route", vp, vp, i, i, i, vp, vp, i, vp)
@@ -118,9 +118,9 @@ def _declare(lib):
     fn("kvcm_moe_grouped_max_tiles", i, i)
     fn("kvcm_moe_grouped", vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp)
     fn("kvcm_pool_update", vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp)
-    fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, f, vp)
+    fn("kvcm_attention_window_pool", vp, i, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, i, f, vp)
     fn("kvcm_attention_window_pool_tiles_supported", i, i, i)
-    fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, i, i, f, vp)
+    fn("kvcm_attention_window_pool_tiles", vp, i, vp, i, vp, vp, vp, vp, vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, f, i, i, i, i, f, vp)
     fn("kvcm_selective_scan", vp, i, i, vp, i, vp, vp, i, i, i, vp, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, i, i, i, vp, C.c_longlong, i, vp)
     fn("kvcm_scan_prepare", vp, i, vp, vp, i, i, i, vp)
     fn("kvcm_delta_prepare", vp, i, vp, i, vp, vp, i, vp, i, vp, vp, vp, vp, i, i, i, vp)
@@ -1207,11 +1207,12 @@ def pool_update(kcache, vcache, pk, pv, tables, table_stride, row_seq, positions
 
 
 def attention_window_pool(q, out, kcache, vcache, pk, pv, tables, table_stride, row_seq, ctx_lens, nh, nkv, d, dv, scale,
-                          window, P, head_scale=None, rows=None, keep_first=0, softcap=0.0, dist_slope=None):
+                          window, P, head_scale=None, rows=None, keep_first=0, softcap=0.0, dist_slope=None, gate=None):
     """out[r, h] = softmax over the last ``window`` tokens, the sequence's first ``keep_first`` tokens and the pooled
     blocks of P tokens before the window (window 0: every token, no blocks) of (q . k) * scale * head_scale[h], times the
     values.  ``softcap`` c > 0: the scores are capped first, c tanh(score / c).  ``dist_slope`` (float32 [nh]): a bias that
-    grows with the distance is taken off the scores, slope[h] * (query position - key position)."""
+    grows with the distance is taken off the scores, slope[h] * (query position - key position).  ``gate`` (float32 rows of
+    >= nh*dv): the output is multiplied element by element with sigmoid(gate) before it is stored."""
     _dev(q, out, kcache, vcache, tables, row_seq, ctx_lens)
     _rows2d(q, "q")
     _rows2d(out, "out")
@@ -1221,11 +1222,15 @@ def attention_window_pool(q, out, kcache, vcache, pk, pv, tables, table_stride, 
     B, E = _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P)
     _f32(head_scale, "head_scale", nh)
     _f32(dist_slope, "dist_slope", nh)
+    if gate is not None:
+        _f32rows(gate, "gate", nh * dv)
+        _need(gate.shape[0] >= T, "attention_window_pool: the gate has fewer rows than the step")
     _i32(row_seq, "row_seq", T)
     _i32(ctx_lens, "ctx_lens", T)
     _i32(tables, "tables")
     _call("kvcm_attention_window_pool", _ptr(q), _DT[q.dtype], q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache),
-          _ptr(pk), _ptr(pv), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), _ptr(head_scale), _ptr(dist_slope), T, nh, nkv, d, dv,
+          _ptr(pk), _ptr(pv), _ptr(tables), table_stride, _ptr(row_seq), _ptr(ctx_lens), _ptr(head_scale), _ptr(dist_slope), _ptr(gate),
+          gate.stride(0) if gate is not None else 0, T, nh, nkv, d, dv,
           B, float(scale), int(window), int(P), E, int(keep_first), float(softcap or 0.0), _stream())
 
 
@@ -1235,7 +1240,7 @@ def attention_window_pool_tiles_supported(d, dv, dtype, block_size):
 
 
 def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_stride, run_start, seq_start, num_seqs, max_run,
-                                nh, nkv, d, dv, scale, window, P, head_scale=None, keep_first=0, softcap=0.0, dist_slope=None):
+                                nh, nkv, d, dv, scale, window, P, head_scale=None, keep_first=0, softcap=0.0, dist_slope=None, gate=None):
     """``attention_window_pool`` for steps whose sequences run several consecutive positions: 64 rows of a run and one
     head per workgroup on the matrix cores (bfloat16 only).  Every row of every run is computed, single rows too."""
     _dev(q, out, kcache, vcache, tables, run_start, seq_start)
@@ -1246,11 +1251,15 @@ def attention_window_pool_tiles(q, out, kcache, vcache, pk, pv, tables, table_st
     B, E = _check_pool(kcache, vcache, pk, pv, nkv, d, dv, P)
     _f32(head_scale, "head_scale", nh)
     _f32(dist_slope, "dist_slope", nh)
+    if gate is not None:
+        _f32rows(gate, "gate", nh * dv)
+        _need(gate.shape[0] >= out.shape[0], "attention_window_pool_tiles: the gate has fewer rows than the output")
     _i32(run_start, "run_start", num_seqs + 1)
     _i32(seq_start, "seq_start", num_seqs)
     _i32(tables, "tables")
     _call("kvcm_attention_window_pool_tiles", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(kcache), _ptr(vcache), _ptr(pk),
-          _ptr(pv), _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), _ptr(head_scale), _ptr(dist_slope), num_seqs, max_run, nh, nkv,
+          _ptr(pv), _ptr(tables), table_stride, _ptr(run_start), _ptr(seq_start), _ptr(head_scale), _ptr(dist_slope), _ptr(gate),
+          gate.stride(0) if gate is not None else 0, num_seqs, max_run, nh, nkv,
           d, dv, B, float(scale), int(window), int(P), E, int(keep_first), float(softcap or 0.0), _stream())
 
 
@@ -1539,13 +1548,23 @@ def gemm_heads(x, w, out, gate=None, rows=None):
 
 
 def act_rows(x, out, activation):
-    """out[T, I] = act(x[T, :I]) for 32-bit rows; act: "silu", "relu" or "gelu_tanh"."""
+    """out[T, I] = act(x[T, :I]) for 32-bit rows (a tensor, or PartialSums whose slices are added first); act: "silu",
+    "relu" or "gelu_tanh"."""
     T, I = out.shape
-    _f32rows(x, "x", I)
     _rows2d(out, "out")
-    _need(x.shape[0] >= T and out.is_cuda, "act_rows: the rows do not agree")
+    splits, stride = 1, 0
+    if isinstance(x, PartialSums):
+        _need(x.rows == T and x.cols == I, "act_rows: the partial sums do not match the output")
+        x, splits, stride = x.data, x.splits, T * I
+        _f32(x, "x", splits * T * I)
+        ld = I
+    else:
+        _f32rows(x, "x", I)
+        _need(x.shape[0] >= T, "act_rows: the rows do not agree")
+        ld = x.stride(0)
+    _need(out.is_cuda, "act_rows: the output must live on the GPU")
     _need(activation in GATE_ACTIVATIONS, f"unknown activation {activation!r} ({sorted(GATE_ACTIVATIONS)})")
-    _call("kvcm_act_rows", _ptr(x), x.stride(0), _ptr(out), _DT[out.dtype], out.stride(0), T, I, GATE_ACTIVATIONS[activation], _stream())
+    _call("kvcm_act_rows", _ptr(x), ld, splits, stride, _ptr(out), _DT[out.dtype], out.stride(0), T, I, GATE_ACTIVATIONS[activation], _stream())
     return out
 
 

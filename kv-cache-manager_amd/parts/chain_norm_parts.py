@@ -184,7 +184,7 @@ class PlainFeedForward(FeedForward):
 
     def forward(self, step, h):
         I, ops = self.params["intermediate_size"], self.ctx.ops
-        up = linear32(self.ctx, step, h, self.w["w_up"], "plain_up")
+        up = linear32(self.ctx, step, h, self.w["w_up"], "plain_up", keep_partial=True)      # slices are added by the activation's launch
         act = step.ws("plain_act", (step.rows, I))
         ops.act_rows(up, act, self.params.get("activation", "gelu_tanh"))
         return linear32(self.ctx, step, act, self.w["w_down"], "plain_out", keep_partial=True)      # the stream's next norm adds the slices

@@ -117,22 +117,26 @@ def _pad_rows(t, multiple=16):
     return torch.cat([t, torch.zeros(extra, t.shape[1], dtype=t.dtype, device=t.device)], 0)
 
 
-def _attend(mixer, step, q, attn, kc, vc, g, nh, nkv, d, dv, scale, window, keep_first=0, softcap=0.0, dist_slope=None):
+def _attend(mixer, step, q, attn, kc, vc, g, nh, nkv, d, dv, scale, window, keep_first=0, softcap=0.0, dist_slope=None, gate=None):
     """Keys and values of one size, no window, no cap on the scores, bfloat16: the kernels every attention over paged
     keys and values takes (parts/paged_attention.py: partitioned for single rows, tiled for runs of positions).
     Otherwise the window attention's: steps with runs of positions take its matrix-core kernel where it has the head
-    shape, others one (row, head) per workgroup."""
+    shape, others one (row, head) per workgroup.  ``gate`` (32-bit logits, one per element of the output): the window
+    attention's kernels multiply their output with its sigmoid as they store it; -> True when that was done (False: the
+    caller still has to)."""
     ops = mixer.ctx.ops
     if d == dv and window == 0 and not softcap and dist_slope is None and attn.dtype == torch.bfloat16 and d % 8 == 0 and d <= 256:
-        return paged_attention.attend(step, ops, q, attn, kc, vc, g, nh, nkv, d, scale, 0)
+        paged_attention.attend(step, ops, q, attn, kc, vc, g, nh, nkv, d, scale, 0)
+        return False
     if step.max_run > 1 and ops.attention_window_pool_tiles_supported(d, dv, attn.dtype, kc.shape[2]):
         ops.attention_window_pool_tiles(q, attn, kc, vc, None, None, step.tables(g), step.table_stride(g), step.run_start,
                                         step.seq_start, step.seqs, step.max_run, nh, nkv, d, dv, scale, window, 0,
-                                        keep_first=keep_first, softcap=softcap, dist_slope=dist_slope)
+                                        keep_first=keep_first, softcap=softcap, dist_slope=dist_slope, gate=gate)
     else:
         ops.attention_window_pool(q, attn, kc, vc, None, None, step.tables(g), step.table_stride(g), step.row_seq, step.ctx_lens,
                                   nh, nkv, d, dv, scale, window, 0, rows=step.rows, keep_first=keep_first, softcap=softcap,
-                                  dist_slope=dist_slope)
+                                  dist_slope=dist_slope, gate=gate)
+    return gate is not None
 
 
 @MIXERS.register("gated_attention")
@@ -494,9 +498,10 @@ class HeadNormWindowAttention(Mixer):
                             bias=w.get("b_proj"), positions=step.positions, temp_coef=self.temp_coef, temp_every=self.temp_every,
                             values_are_keys=self.values == "keys", slots=slots, kcache=kc, vcache=vc, rows=T)
         attn = step.ws("hwa_attn", (T, self.nh * self.dv))
-        _attend(self, step, q, attn, kc, vc, g, self.nh, self.nkv, self.d, self.dv, p["scale"], self.window,
-                dist_slope=w.get("slopes"))
-        if self.gate:
-            ops.head_gate(attn, proj[:, self.gate_at:], self.nh, self.dv, rows=T, per_element=True)
+        gate = proj[:, self.gate_at:] if self.gate else None
+        gated = _attend(self, step, q, attn, kc, vc, g, self.nh, self.nkv, self.d, self.dv, p["scale"], self.window,
+                        dist_slope=w.get("slopes"), gate=gate)
+        if self.gate and not gated:
+            ops.head_gate(attn, gate, self.nh, self.dv, rows=T, per_element=True)
         out = linear32(self.ctx, step, attn, w["w_o"], "hwa_out", keep_partial=True)      # the stream's next norm adds the slices
         return ops.BiasedOutput(out, w["b_o"]) if self.bias else out

@@ -169,6 +169,17 @@ def test_window_attention_with_a_distance_bias_and_keys_that_stand_out_at_every_
                 ops.attention_window_pool_tiles(qd, out2, kc, vc, None, None, tables, len(table), st.run_start, st.seq_start, 1, n - first,
                                                 nh, nkv, d, dv, scale, W, 0, dist_slope=dev(slopes))
                 np.testing.assert_allclose(out2.float().cpu().numpy(), want[first:].reshape(n - first, -1), atol=tol, err_msg=f"tiles: key {spot} rows from {first}")
+    # a gate per element in the kernels' epilogue (the inputs of the loop's last round: every row of the sequence as one run)
+    gate = rng.normal(size=(n - first, nh * dv + 3)) * 2
+    gated = want[first:].reshape(n - first, -1) * plain.logistic(gate[:, :nh * dv])
+    out4 = torch.empty_like(out)
+    ops.attention_window_pool(qd, out4, kc, vc, None, None, tables, len(table), st.row_seq, st.ctx_lens, nh, nkv, d, dv, scale, W, 0,
+                              dist_slope=dev(slopes), gate=dev(gate))
+    np.testing.assert_allclose(out4.float().cpu().numpy(), gated, atol=tol)
+    if ops.attention_window_pool_tiles_supported(d, dv, dtype, B):
+        ops.attention_window_pool_tiles(qd, out4, kc, vc, None, None, tables, len(table), st.run_start, st.seq_start, 1, n - first,
+                                        nh, nkv, d, dv, scale, W, 0, dist_slope=dev(slopes), gate=dev(gate))
+        np.testing.assert_allclose(out4.float().cpu().numpy(), gated, atol=tol)
     # the bias matters: without it the same inputs give another answer
     out3 = torch.empty_like(out)
     ops.attention_window_pool(qd, out3, kc, vc, None, None, tables, len(table), st.row_seq, st.ctx_lens, nh, nkv, d, dv, scale, W, 0)
@@ -236,6 +247,14 @@ def test_rotation_with_keys_and_values_in_rows_of_their_own():
             np.testing.assert_allclose(kc[s // B, 0, s % B].cpu().numpy(), want_k[t], atol=2e-6)
             np.testing.assert_allclose(vc[s // B, 0, :, s % B].cpu().numpy(), kv[t, 7 + dk:], atol=1e-6)
     assert float(kc.abs().sum(-1).gt(0).sum()) == 5
+    # steps of few rows take a workgroup per head, steps of many one per row: the same bits
+    many = 4
+    q_big = torch.empty(many * T, nh * dk, device=DEV)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ops.rotate_store(dev(np.tile(q, (many, 1))), q_big, nh, 1, dk, r, cos_sin=table.repeat(many, 1), rot=dims,
+                     slots=torch.cat([slots] + [torch.full_like(slots, -1)] * (many - 1)), kcache=kc2, vcache=vc2, halves=True,
+                     kv=dev(np.tile(kv, (many, 1)))[:, 7:])
+    assert torch.equal(q_big[:T], q_out) and torch.equal(q_big[-T:], q_out) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
     # a layer that only reads pages: queries alone, nothing stored
     q_only = torch.empty(T, nh * dk, device=DEV)
     ops.rotate_store(dev(q)[:, :nh * dk].contiguous(), q_only, nh, 1, dk, r, cos_sin=table, rot=dims, halves=True)
@@ -278,6 +297,10 @@ def test_small_elementwise_pieces():
         z = rng.normal(size=(T, 37)) * 3
         act = torch.empty(T, 33, dtype=dt, device=DEV)
         ops.act_rows(dev(z), act, "gelu_tanh")
+        np.testing.assert_allclose(act.float().cpu().numpy(), plain.gelu_tanh(z[:, :33]), atol=tol * 12)
+        parts = rng.normal(size=(3, T, 33))      # the slices of a split product are added on the way
+        parts[0] = z[:, :33] - parts[1:].sum(0)
+        ops.act_rows(ops.PartialSums(dev(parts), 3, T, 33, torch.empty(T, 33, device=DEV)), act, "gelu_tanh")
         np.testing.assert_allclose(act.float().cpu().numpy(), plain.gelu_tanh(z[:, :33]), atol=tol * 12)
         x, w = rng.normal(size=(T, 50)), 1.0 + 0.1 * rng.normal(size=20)
         xs, out = dev(x), torch.zeros(T, 24, dtype=dt, device=DEV)
