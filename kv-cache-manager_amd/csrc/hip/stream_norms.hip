@@ -87,12 +87,35 @@ __global__ void __launch_bounds__(256)
   if (item >= items) return;
   const int lane = threadIdx.x % kWave;
   float* p = x + (item / groups) * ld + col0 + (item % groups) * size;
+  TO* q = out ? out + (item / groups) * ldo + (item % groups) * size : nullptr;
+  constexpr int kHeld = 16;      // values a lane keeps: groups of up to 1,024 are read once, all loads on their way together
+  if (size <= kHeld * kWave) {
+    float v[kHeld];
+#pragma unroll
+    for (int j = 0; j < kHeld; ++j) {
+      const int i = lane + j * kWave;
+      v[j] = i < size ? p[i] : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < kHeld; ++j) ss = fmaf(v[j], v[j], ss);      // (the same order of sums as the loop below: lane, then j)
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / float(size) + eps);
+#pragma unroll
+    for (int j = 0; j < kHeld; ++j) {
+      const int i = lane + j * kWave;
+      if (i >= size) break;
+      const float y = v[j] * inv * w[i];
+      if (q) store_f(q + i, y);
+      else p[i] = y;
+    }
+    return;
+  }
   float ss = 0.f;
   for (int i = lane; i < size; i += kWave) ss = fmaf(p[i], p[i], ss);
   ss = wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / float(size) + eps);
-  if (out) {
-    TO* q = out + (item / groups) * ldo + (item % groups) * size;
+  if (q) {
     for (int i = lane; i < size; i += kWave) store_f(q + i, p[i] * inv * w[i]);
   } else {
     for (int i = lane; i < size; i += kWave) p[i] = p[i] * inv * w[i];
