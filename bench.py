@@ -222,7 +222,7 @@ def fisesun_config(width, layers, vocab=32000):
 
 
 # Betirax at a width: (cached latent, rotated key part, query latent, positions per temperature step, experts, experts a row)
-BETIRAX_SIZES = {2048: (96, 32, 768, 1024, 8, 2), 4096: (96, 32, 1536, 1024, 8, 2)}
+BETIRAX_SIZES = {2048: (64, 64, 768, 1024, 8, 2), 4096: (64, 64, 1536, 1024, 8, 2)}
 
 
 def betirax_config(width, layers, vocab=32000):
@@ -236,7 +236,7 @@ def betirax_config(width, layers, vocab=32000):
     moe = {"kind": "moe", "expert": {"ff": ff // (2 * top)}, "router": {"experts": experts, "top": top}, "shared": {"ff": ff // 2}}
     dense = {"kind": "dense", "ff": ff}
     attention = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": window},
-                 "q_temp": {"coef": 0.5, "every": every}}
+                 "q_temp": {"coef": 0.25, "every": every}}
     latent = {"heads": nh, "dim": hd, "rot_dim": rot, "vdim": hd, "kv_rank": rank, "q_rank": q_rank, "scale": (hd + rot) ** -0.5,
               "rot": {"dims": rot, "base": 10000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
     listed, owner = [], None
@@ -252,7 +252,7 @@ def betirax_config(width, layers, vocab=32000):
         else:
             listed.append({"type": "attention", "mixer": attention, "mlp": mlp})
     return BetiraxConfig.from_dict({"architecture": "Betirax", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
-                                    "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "layers": listed})
+                                    "norm": {"eps": 1e-6}, "postln_alpha": 2.0, "layers": listed})
 
 
 def design_main(args):
