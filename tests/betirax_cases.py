@@ -6,7 +6,7 @@ for all, a rotated key part that is absent, partly and wholly rotated, with and 
 matrix-core kernels take and sizes that they refuse, windows of one token, shorter and longer than a page and none,
 query temperatures whose steps are shorter and longer than a page and none, a stream factor of one (left out of the
 file) and others, and layers that read an earlier layer's pages right after it and several layers later, two of them the
-same layer's.
+same layer's, and sizes of which none is a multiple of 8.
 """
 import numpy as np
 import torch
@@ -50,6 +50,7 @@ def _layer(mixer, mlp=None):
 
 _ROT_P = dict(dims=4, base=100.0, scaling=(3.0, 40, 4.0, 1.0))
 _ROT_Q = dict(dims=32, base=5000.0, scaling=(8.0, 256, 16.0, 2.0))
+_ROT_T = dict(dims=12, base=30000.0, scaling=(6.0, 512, 20.0, 1.5))
 CONFIGS = {
     # a latent attention first whose pages the third layer reads; odd head sizes off the multiples of 8; a layer without a
     # feed-forward; expert sizes off the multiples of 16; temperature steps shorter than a page
@@ -78,8 +79,14 @@ CONFIGS = {
     "S": {"architecture": "Betirax", "vocab": 200, "width": 96, "embedding": {"scale": 0.5}, "norm": {"eps": 1e-5}, "postln_alpha": 3.0,
           "layers": [_layer(_attention(6, 2, 128, 0.09, window=70, temp=(0.25, 64)), _moe(8, 3, 48, shared=64)),
                      _layer(_latent(2, 48, 16, 24, 40, 56, 0.15, base=25000.0), _dense(64))]},
+    # nothing a multiple of 8: a width of 100, an odd vocabulary, five heads of 20, latents of 36 beside a rotated part of 12
+    "T": {"architecture": "Betirax", "vocab": 451, "width": 100, "embedding": {"scale": 7.0}, "norm": {"eps": 1e-5}, "postln_alpha": 2.2,
+          "layers": [_layer(_attention(5, 5, 20, 0.2, window=23, temp=(0.7, 30)), _dense(150)),
+                     _layer(_latent(3, 20, 12, 28, 36, 44, 0.17, **_ROT_T), _moe(6, 3, 50, shared=70)),
+                     _layer(_attention(6, 3, 12, 0.25, window=64, temp=(0.2, 7)), _moe(3, 2, 33)),
+                     _layer(_latent(5, 10, 12, 14, 36, 21, 0.2, kv_from=1, **_ROT_T), _dense(77))]},
 }
-BLOCK_SIZE = {"P": 16, "Q": 16, "R": 8, "S": 32}
+BLOCK_SIZE = {"P": 16, "Q": 16, "R": 8, "S": 32, "T": 16}
 
 
 def tensors_for(raw, seed, sharpen=3.0):
