@@ -239,7 +239,8 @@ int kvcm_mlstm_scan(const float* q, int ldq, const float* k, int ldk, const floa
                     const int* seq_start, const int* state_slots, int S, int heads, int dk, int dv, int T, int max_run,
                     hipStream_t s);
 // (moe.hip) a routed feed-forward: the choice of experts, and the experts' two products a row at a time
-int kvcm_moe_route(const float* logits, int ld, int E, int top, int over_chosen, int* chosen, float* weight, int T, hipStream_t s);
+int kvcm_moe_route(const float* logits, int ld, int splits, long long split_stride, int E, int top, int over_chosen, int* chosen,
+                   float* weight, int T, hipStream_t s);
 int kvcm_moe_table_route(const int* tokens, const int* table, int vocab, int ld, int top, int* chosen, float* weight, int T,
                          hipStream_t s);
 int kvcm_moe_up(const void* h, int dtype, int ldh, const void* w_up, const int* chosen, void* act, int T, int K, int F, int top,

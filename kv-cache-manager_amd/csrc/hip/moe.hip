@@ -23,13 +23,23 @@
 namespace kvcm {
 
 constexpr int kMoeMaxTop = 16;
+constexpr int kMoeMaxExperts = 1024;      // a row's logits are kept in LDS while its experts are picked
 
 __global__ void __launch_bounds__(256)
-    moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top, int over_chosen, int* __restrict__ chosen,
-                     float* __restrict__ weight, int T) {
+    moe_route_kernel(const float* __restrict__ logits, int ld, int splits, size_t split_stride, int E, int top, int over_chosen,
+                     int* __restrict__ chosen, float* __restrict__ weight, int T) {
+  // up to 64 experts a lane group: the row's logits are formed once (a router product that was split along K arrives as
+  // slices, which are added here in their order) and kept in LDS
+  __shared__ float zs[256 / kWave][kMoeMaxExperts];
   const int row = blockIdx.x * (256 / kWave) + threadIdx.x / kWave, lane = threadIdx.x % kWave;
   if (row >= T) return;
-  const float* z = logits + size_t(row) * ld;
+  float* z = zs[threadIdx.x / kWave];
+  for (int e = lane; e < E; e += kWave) {
+    float v = logits[size_t(row) * ld + e];
+    for (int sl = 1; sl < splits; ++sl) v += logits[size_t(sl) * split_stride + size_t(row) * ld + e];
+    z[e] = v;
+  }
+  __builtin_amdgcn_wave_barrier();
   float mx = -FLT_MAX;
   for (int e = lane; e < E; e += kWave) mx = fmaxf(mx, z[e]);
   mx = wave_max(mx);
@@ -220,11 +230,14 @@ using namespace kvcm;
 
 extern "C" {
 
-int kvcm_moe_route(const float* logits, int ld, int E, int top, int over_chosen, int* chosen, float* weight, int T, hipStream_t s) {
+int kvcm_moe_route(const float* logits, int ld, int splits, long long split_stride, int E, int top, int over_chosen, int* chosen,
+                   float* weight, int T, hipStream_t s) {
   if (T == 0) return 0;
   KVCM_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E && ld >= E, "moe_route: bad sizes T=%d experts=%d top=%d", T, E, top);
   KVCM_REQUIRE(top <= kMoeMaxTop, "moe_route: %d experts a row are not supported (up to %d)", top, kMoeMaxTop);
-  moe_route_kernel<<<(T + 3) / 4, 256, 0, s>>>(logits, ld, E, top, over_chosen, chosen, weight, T);
+  KVCM_REQUIRE(E <= kMoeMaxExperts, "moe_route: %d experts are not supported (up to %d)", E, kMoeMaxExperts);
+  KVCM_REQUIRE(splits >= 1 && split_stride >= 0, "moe_route: the logits have at least one slice");
+  moe_route_kernel<<<(T + 3) / 4, 256, 0, s>>>(logits, ld, splits, static_cast<size_t>(split_stride), E, top, over_chosen, chosen, weight, T);
   return launch_status("moe_route");
 }
 

@@ -18,13 +18,25 @@ namespace kvcm {
 
 constexpr int kPostThreads = 256;
 
+// Sum over the workgroup's four waves with one barrier: every thread adds the waves' sums itself, in wave order.  Each
+// reduction of a kernel brings a scratch array of its own, so that none has to wait for the readers of the one before.
+__device__ __forceinline__ float post_block_sum(float v, float* scratch /* kPostThreads / 64 floats, not shared with another sum */) {
+  v = wave_sum(v);
+  if (threadIdx.x % kWave == 0) scratch[threadIdx.x / kWave] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int w = 0; w < kPostThreads / kWave; ++w) s += scratch[w];
+  return s;
+}
+
 // any row length: the row is formed three times from its sources (mean, deviations, result)
 template <class TO>
 __global__ void __launch_bounds__(kPostThreads)
     layernorm_post_kernel(float* __restrict__ x, const float* __restrict__ a, int a_splits, size_t split_stride,
                           const float* __restrict__ bias, float alpha, const float* __restrict__ w,
                           const int* __restrict__ rows, TO* __restrict__ out, int H, float eps) {
-  __shared__ float scratch[kPostThreads / kWave + 1];
+  __shared__ float scratch_mean[kPostThreads / kWave], scratch_var[kPostThreads / kWave];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   float* xr = x + size_t(src) * H;
@@ -42,13 +54,14 @@ __global__ void __launch_bounds__(kPostThreads)
   const float inv_h = 1.0f / float(H);
   float sum = 0.f;
   for (int i = threadIdx.x; i < H; i += kPostThreads) sum += value(i);
-  const float mean = block_sum<kPostThreads>(sum, scratch) * inv_h;
+  const float mean = post_block_sum(sum, scratch_mean) * inv_h;
   float sq = 0.f;
   for (int i = threadIdx.x; i < H; i += kPostThreads) {
     const float c = value(i) - mean;
     sq = fmaf(c, c, sq);
   }
-  const float inv = 1.0f / sqrtf(block_sum<kPostThreads>(sq, scratch) * inv_h + eps);
+  const float inv = 1.0f / sqrtf(post_block_sum(sq, scratch_var) * inv_h + eps);
+  __syncthreads();      // nobody writes the stream before everybody has read it for the last statistic
   for (int i = threadIdx.x; i < H; i += kPostThreads) {
     const float y = (value(i) - mean) * inv * w[i];
     if (!rows) xr[i] = y;      // each element is read and written by one thread only
@@ -62,7 +75,7 @@ __global__ void __launch_bounds__(kPostThreads)
     layernorm_post_rows_kernel(float* __restrict__ x, const float* __restrict__ a, int a_splits, size_t split_stride,
                                const float* __restrict__ bias, float alpha, const float* __restrict__ w,
                                const int* __restrict__ rows, TO* __restrict__ out, int H, float eps) {
-  __shared__ float scratch[kPostThreads / kWave + 1];
+  __shared__ float scratch_mean[kPostThreads / kWave], scratch_var[kPostThreads / kWave];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   float* xr = x + size_t(src) * H;
@@ -97,7 +110,7 @@ __global__ void __launch_bounds__(kPostThreads)
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       if (in[g]) sum += v[g][e];
-  const float mean = block_sum<kPostThreads>(sum, scratch) * inv_h;
+  const float mean = post_block_sum(sum, scratch_mean) * inv_h;
   float sq = 0.f;
 #pragma unroll
   for (int g = 0; g < G; ++g)
@@ -106,7 +119,7 @@ __global__ void __launch_bounds__(kPostThreads)
       v[g][e] -= mean;
       if (in[g]) sq = fmaf(v[g][e], v[g][e], sq);
     }
-  const float inv = 1.0f / sqrtf(block_sum<kPostThreads>(sq, scratch) * inv_h + eps);
+  const float inv = 1.0f / sqrtf(post_block_sum(sq, scratch_var) * inv_h + eps);
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     if (!in[g]) continue;

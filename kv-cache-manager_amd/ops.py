@@ -110,7 +110,7 @@ def _declare(lib):
     fn("kvcm_gemm_heads", vp, i, i, vp, vp, i, i, vp, i, i, i, i, i, vp)
     fn("kvcm_act_rows", vp, i, i, C.c_longlong, vp, i, i, i, i, i, vp)
     fn("kvcm_mlstm_scan", vp, i, vp, i, vp, i, vp, i, vp, i, vp, vp, f, f, vp, vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp)
-    fn("kvcm_moe_route", vp, i, i, i, i, vp, vp, i, vp)
+    fn("kvcm_moe_route", vp, i, i, C.c_longlong, i, i, i, vp, vp, i, vp)
     fn("kvcm_moe_table_route", vp, vp, i, i, i, vp, vp, i, vp)
     fn("kvcm_moe_up", vp, i, i, vp, vp, vp, i, i, i, i, i, i, vp)
     fn("kvcm_moe_down", vp, i, vp, vp, vp, vp, vp, i, i, i, i, i, vp)
@@ -1593,14 +1593,24 @@ def mlstm_scan(q, k, v, gate_in, gate_keep, in_bias, keep_bias, cap, q_scale, co
 def moe_route(logits, experts, top, chosen, weight, rows=None, over_chosen=False):
     """chosen[T, top] (int32) and weight[T, top] (float32): the ``top`` experts with the largest softmax scores over all
     ``experts`` of each row's 32-bit router logits, best first, with those scores; ``over_chosen``: with the softmax over
-    the chosen logits alone instead (the weights of a row add up to one)."""
+    the chosen logits alone instead (the weights of a row add up to one).  ``logits`` may be PartialSums (a router product
+    that was split along K): the slices are added as they are read."""
     T = chosen.shape[0] if rows is None else rows
-    _f32rows(logits, "logits", experts)
+    splits, stride = 1, 0
+    if isinstance(logits, PartialSums):
+        _need(logits.rows >= T and logits.cols >= experts, "moe_route: the partial sums do not hold the rows' logits")
+        splits, stride, ld, logits = logits.splits, logits.rows * logits.cols, logits.cols, logits.data
+        _f32(logits, "logits", splits * stride)
+    else:
+        _f32rows(logits, "logits", experts)
+        _need(logits.shape[0] >= T, "moe_route: fewer rows of logits than rows")
+        ld = logits.stride(0)
     _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.is_cuda and chosen.shape[1] == top and chosen.shape[0] >= T,
           "chosen must be int32 [T, top]")
     _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.is_cuda and tuple(weight.shape) == tuple(chosen.shape),
           "weight must be float32 [T, top]")
-    _call("kvcm_moe_route", _ptr(logits), logits.stride(0), experts, top, 1 if over_chosen else 0, _ptr(chosen), _ptr(weight), T, _stream())
+    _call("kvcm_moe_route", _ptr(logits), ld, splits, stride, experts, top, 1 if over_chosen else 0, _ptr(chosen), _ptr(weight),
+          T, _stream())
 
 
 def moe_table_route(tokens, table, top, chosen, weight, rows=None):

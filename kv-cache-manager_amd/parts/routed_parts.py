@@ -113,7 +113,7 @@ class RoutedExperts(FeedForward):
         if self.routing == "table":
             ops.moe_table_route(step.tokens, w["table"], top, chosen, weight, rows=T)
         else:
-            logits = linear32(self.ctx, step, h, w["w_router"], "routed_logits")
+            logits = linear32(self.ctx, step, h, w["w_router"], "routed_logits", keep_partial=True)      # the route adds the slices
             ops.moe_route(logits, E, top, chosen, weight, rows=T, over_chosen=self.routing == "softmax_chosen")
         add = self.shared.forward(step, h) if self.shared is not None else None      # 32-bit [T, H]: the experts' sum starts from it
         H = self.ctx.hidden_size

@@ -315,6 +315,11 @@ def test_small_elementwise_pieces():
         assert chosen.cpu().numpy().tolist() == want_c.tolist()
         np.testing.assert_allclose(weight.cpu().numpy(), want_w, atol=2e-6)
         np.testing.assert_allclose(weight.sum(-1).cpu().numpy(), 1.0, atol=1e-6)
+        parts = rng.normal(size=(3, 9, E))      # a router product that was split along K: the route adds its slices
+        parts[0] = z - parts[1:].sum(0)
+        ops.moe_route(ops.PartialSums(dev(parts), 3, 9, E, torch.empty(9, E, device=DEV)), E, top, chosen, weight, over_chosen=True)
+        assert chosen.cpu().numpy().tolist() == want_c.tolist()
+        np.testing.assert_allclose(weight.cpu().numpy(), want_w, atol=1e-5)
 
 
 # ------------------------------------------------------------------------------ whole models
