@@ -238,7 +238,7 @@ def betirax_config(width, layers, vocab=32000):
     attention = {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": window},
                  "q_temp": {"coef": 0.25, "every": every}}
     latent = {"heads": nh, "dim": hd, "rot_dim": rot, "vdim": hd, "kv_rank": rank, "q_rank": q_rank, "scale": (hd + rot) ** -0.5,
-              "rot": {"dims": rot, "base": 10000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+              "rot": {"dims": rot, "base": 10000.0, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
     listed, owner = [], None
     for i in range(layers):
         mlp = dense if i % 2 == 0 else moe
